@@ -1,0 +1,65 @@
+"""Builds hqmq_amd/libhqmq_amd.so from hqmq_amd/csrc/*.hip with hipcc for gfx950.
+
+    python -m hqmq_amd.build            # compile (always) and link
+
+The kernels that decide integers (codeword index, radius code, Med3x mask) are
+compiled with -ffp-contract=off so that every written float operation rounds
+on its own; the attention kernels keep the default contraction.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+OUT = HERE / "libhqmq_amd.so"
+
+COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+EXACT = {"joint.hip", "quantize.hip", "med3x.hip", "dequant.hip"}
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found; libhqmq_amd.so cannot be built")
+    return exe
+
+
+def build(verbose: bool = False) -> Path:
+    cc = hipcc()
+    objdir = HERE / "build"
+    objdir.mkdir(exist_ok=True)
+    srcs = sorted(CSRC.glob("*.hip"))
+    if not srcs:
+        raise RuntimeError(f"no sources under {CSRC}")
+
+    def compile_one(src: Path) -> Path:
+        obj = objdir / (src.stem + ".o")
+        cmd = [cc, *COMMON, "-c", str(src), "-o", str(obj)]
+        if src.name in EXACT:
+            cmd.insert(1, "-ffp-contract=off")
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if verbose or r.returncode:
+            sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+        if r.returncode:
+            raise RuntimeError(f"hipcc failed on {src.name}")
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
+        objs = list(ex.map(compile_one, srcs))
+    cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode:
+        sys.stderr.write(r.stdout + r.stderr)
+        raise RuntimeError("link failed")
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

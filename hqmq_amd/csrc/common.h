@@ -1,0 +1,84 @@
+// Shared device helpers for the HQMQ kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/hqmq_amd.h"
+
+#define HQMQ_VERSION 0x000100
+
+namespace hqmq {
+
+constexpr int kWave = 64;
+constexpr int kTile = 16;  // tokens per sideband tile / MFMA tile
+
+// ---- bit-exact conversions: fp32 <-> D with round-to-nearest-even ----------
+struct F32 {
+    using storage = float;
+    static constexpr int code = HQMQ_F32;
+    static __device__ __forceinline__ float load(const storage *p) { return *p; }
+    static __device__ __forceinline__ void store(storage *p, float f) { *p = f; }
+    static __device__ __forceinline__ float rnd(float f) { return f; }
+    static __device__ __forceinline__ float eps() { return 5.9604645e-8f; }  // 2^-24
+};
+struct F16 {
+    using storage = uint16_t;
+    static constexpr int code = HQMQ_F16;
+    static __device__ __forceinline__ float load(const storage *p) { return __half2float(__ushort_as_half(*p)); }
+    static __device__ __forceinline__ void store(storage *p, float f) { *p = __half_as_ushort(__float2half_rn(f)); }
+    static __device__ __forceinline__ float rnd(float f) { return __half2float(__float2half_rn(f)); }
+    static __device__ __forceinline__ float eps() { return 4.8828125e-4f; }  // 2^-11
+};
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+    return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+struct BF16 {
+    using storage = uint16_t;
+    static constexpr int code = HQMQ_BF16;
+    static __device__ __forceinline__ float load(const storage *p) { return __uint_as_float((uint32_t)(*p) << 16); }
+    static __device__ __forceinline__ void store(storage *p, float f) { *p = f32_to_bf16_bits(f); }
+    static __device__ __forceinline__ float rnd(float f) { return __uint_as_float((uint32_t)f32_to_bf16_bits(f) << 16); }
+    static __device__ __forceinline__ float eps() { return 3.90625e-3f; }  // 2^-8
+};
+
+__device__ __forceinline__ bool is_nan(float f) { return f != f; }
+
+// torch clamp(min=c) on a D tensor: NaN propagates, the bound is rounded to D.
+template <class D>
+__device__ __forceinline__ float clamp_min_d(float v, float lo_f32) {
+    if (is_nan(v)) return v;
+    float lo = D::rnd(lo_f32);
+    return v < lo ? lo : v;
+}
+
+// ||chunk||_2 as torch's CPU norm computes it: fp32, products and sums rounded one by one.
+// Built with -ffp-contract=off, so none of these fuse.
+__device__ __forceinline__ float norm4(float a, float b, float c, float d) {
+    float s = a * a;
+    s = s + b * b;
+    s = s + c * c;
+    s = s + d * d;
+    return sqrtf(s);
+}
+
+inline int layout_bits(int S, int radius_bits, int *idx_bits, int *main_bits, int *aux_bits) {
+    if (S < 1 || S > 2730 || radius_bits < 1 || radius_bits > 8) return HQMQ_ERR_SHAPE;
+    int K = 24 * S, ib = 0;
+    while ((1 << ib) < K) ib++;
+    int cb = ib + radius_bits;
+    int mb = 4 * (cb / 4);
+    if (mb < 8) mb = 8;
+    if (mb > 16) mb = 16;
+    int ab = cb > mb ? cb - mb : 0;
+    if (idx_bits) *idx_bits = ib;
+    if (main_bits) *main_bits = mb;
+    if (aux_bits) *aux_bits = ab;
+    return HQMQ_OK;
+}
+
+inline int hip_status(hipError_t e) { return e == hipSuccess ? HQMQ_OK : (int)e; }
+
+}  // namespace hqmq

@@ -1,0 +1,338 @@
+// HQMQ quantize (+ Med3x mask, + bit-packing) for one K or V tensor.
+//
+// Follows HQMQQuantizer._qdq, unit-magnitude / linear-radius branch
+// (src/quantizers/hqmq.py:145-158,164-169,208-216 of the reference) and the
+// mask/merge of OutlierAwareHQMQQuantizer._qdq (src/quantizers/outlier_aware.py:72,86).
+//
+// One lane per 4-element chunk.  The codeword the reference picks is
+//     first k = p*S+s maximising  RNE_D( fma-chain_fp32( u . J[k] ) ),
+// u = RNE_D(x / r).  Instead of scoring all 24*S rows, each lane rotates its
+// chunk by conj(q_s) (q_s broadcast from LDS): <u, q_p*q_s> = <u*conj(q_s), q_p>,
+// and the best Hurwitz unit for a rotated chunk v is closed form
+// (max_i |v_i| for the 8 axis units, sum_i |v_i| / 2 for the 16 half units).
+// That gives the exact-arithmetic score of the best p for every s in ~25
+// operations.  Rounding decides the reference's choice among near-ties, so the
+// closed form is only a filter: every (p, s) whose exact score is within a
+// proven margin of the best is re-scored with the reference's rounding, and
+// the smallest index among the maxima wins.  The margin covers the rounding of
+// the joint table (slack[h] from hqmq_build_joint), the final RNE_D of the
+// score and the float error of the filter itself.  Lanes whose candidate lists
+// overflow, or whose direction is not finite, score all 24*S rows instead.
+//
+// Compiled with -ffp-contract=off; fused multiply-adds are written explicitly.
+#include "common.h"
+
+namespace hqmq {
+
+constexpr int kQThreads = 256;
+constexpr int kSCap = 32;  // candidate secondaries kept per lane
+constexpr int kKCap = 24;  // candidate codewords kept per lane
+
+struct QParams {
+    const void *x;
+    int64_t xsb, xsh, xst;
+    int B, H, T, n;
+    const void *joint;
+    const float *slack;
+    int S, qmax;
+    int32_t *idx_out, *rq_out;
+    void *rmax_out, *dense_out;
+    const void *thr;
+    uint8_t *mask_out;
+    uint8_t *main_plane, *aux_plane, *flag_plane;
+    void *scale_plane;
+    int64_t t_cap;
+    int t_off;
+    const int32_t *pos;
+    int idx_bits, main_bits, aux_bits;
+    int tokens_per_block;
+    int32_t *stats;
+};
+
+__device__ __forceinline__ void rotate_conj(const float u[4], float qw, float qx, float qy, float qz, float v[4]) {
+    // v = u * conj(q)
+    v[0] = fmaf(u[3], qz, fmaf(u[2], qy, fmaf(u[1], qx, u[0] * qw)));
+    v[1] = fmaf(u[3], qy, fmaf(-u[2], qz, fmaf(u[1], qw, -u[0] * qx)));
+    v[2] = fmaf(-u[3], qx, fmaf(u[2], qw, fmaf(u[1], qz, -u[0] * qy)));
+    v[3] = fmaf(u[3], qw, fmaf(u[2], qx, fmaf(-u[1], qy, -u[0] * qz)));
+}
+
+// twice the exact score of the best Hurwitz unit for rotated chunk v
+__device__ __forceinline__ float best2_of(const float v[4]) {
+    float a0 = fabsf(v[0]), a1 = fabsf(v[1]), a2 = fabsf(v[2]), a3 = fabsf(v[3]);
+    float sum = (a0 + a1) + (a2 + a3);
+    float mx = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+    return fmaxf(mx + mx, sum);
+}
+
+// twice the exact score of Hurwitz unit p for rotated chunk v
+__device__ __forceinline__ float exact2_of(const float v[4], int p) {
+    if (p < 8) {
+        float t = v[p >> 1];
+        t = t + t;
+        return (p & 1) ? -t : t;
+    }
+    int m = p - 8;
+    float t0 = (m & 8) ? -v[0] : v[0], t1 = (m & 4) ? -v[1] : v[1];
+    float t2 = (m & 2) ? -v[2] : v[2], t3 = (m & 1) ? -v[3] : v[3];
+    return (t0 + t1) + (t2 + t3);
+}
+
+template <class D>
+__device__ __forceinline__ float ref_score(const float u[4], const typename D::storage *row) {
+    float j0 = D::load(row), j1 = D::load(row + 1), j2 = D::load(row + 2), j3 = D::load(row + 3);
+    float acc = u[0] * j0;
+    acc = fmaf(u[1], j1, acc);
+    acc = fmaf(u[2], j2, acc);
+    acc = fmaf(u[3], j3, acc);
+    return D::rnd(acc);
+}
+
+// argmax over all K rows with torch's rule: first maximum, NaN counts as maximum.
+template <class D>
+__device__ int brute_argmax(const float u[4], const typename D::storage *jh, int K) {
+    int best = 0;
+    float bs = 0.f;
+    for (int k = 0; k < K; k++) {
+        float s = ref_score<D>(u, jh + (size_t)k * 4);
+        if (is_nan(s)) return k;
+        if (k == 0 || s > bs) { bs = s; best = k; }
+    }
+    return best;
+}
+
+// Little-endian bit stream of `w`-bit fields (field i = vals[base + i] >> shift, masked)
+// -> output byte `byte` of the row.
+__device__ __forceinline__ uint8_t gather_byte(const uint32_t *vals, int count, int w, int shift, int byte) {
+    uint32_t out = 0;
+    uint32_t fmask = (w >= 32) ? 0xffffffffu : ((1u << w) - 1u);
+    for (int bit = 0; bit < 8; bit++) {
+        int pos = byte * 8 + bit;
+        int i = pos / w, o = pos - i * w;
+        if (i < count) out |= ((((vals[i] >> shift) & fmask) >> o) & 1u) << bit;
+    }
+    return (uint8_t)out;
+}
+
+template <class D, int ALGO>
+__global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
+    using ST = typename D::storage;
+    extern __shared__ float sec[];  // [S][4]
+    __shared__ float radius_sh[kQThreads];
+    __shared__ uint32_t code_sh[kQThreads];
+    __shared__ uint32_t mask_sh[kQThreads];
+    __shared__ uint16_t slist[kSCap][kQThreads];
+    __shared__ uint16_t klist[kKCap][kQThreads];
+
+    const int tid = threadIdx.x;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
+    const int n = a.n, S = a.S, K = 24 * S;
+    const int tok_local = tid / n, c = tid - tok_local * n;
+    const int t = blockIdx.x * a.tokens_per_block + tok_local;
+    const bool active = tok_local < a.tokens_per_block && t < a.T;
+    const ST *jh = (const ST *)a.joint + (size_t)h * K * 4;
+
+    for (int i = tid; i < S * 4; i += kQThreads) sec[i] = D::load(jh + i);  // rows k = s are q_s itself
+
+    float xv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (active) {
+        const ST *xp = (const ST *)a.x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst + c * 4;
+        for (int j = 0; j < 4; j++) xv[j] = D::load(xp + j);
+    }
+    const float nrm = D::rnd(norm4(xv[0], xv[1], xv[2], xv[3]));
+    const float r = clamp_min_d<D>(nrm, 1e-8f);
+    float u[4];
+    for (int j = 0; j < 4; j++) u[j] = D::rnd(xv[j] / r);
+    radius_sh[tid] = r;
+    __syncthreads();
+
+    // ---- codeword search ----
+    int idx = 0;
+    const bool finite = fabsf(u[0]) < INFINITY && fabsf(u[1]) < INFINITY && fabsf(u[2]) < INFINITY && fabsf(u[3]) < INFINITY;
+    const bool zero = u[0] == 0.f && u[1] == 0.f && u[2] == 0.f && u[3] == 0.f;
+    if (ALGO == 1) {
+        if (active) idx = brute_argmax<D>(u, jh, K);
+    } else {
+        bool brute = active && !finite;            // NaN/inf directions: exact emulation only
+        const bool search = active && finite && !zero;  // all-zero direction: every score is 0 -> index 0
+        float us[4];
+        for (int j = 0; j < 4; j++) us[j] = search ? u[j] : (j == 0 ? 1.f : 0.f);
+        const float ulen = sqrtf(fmaf(us[3], us[3], fmaf(us[2], us[2], fmaf(us[1], us[1], us[0] * us[0])))) * 1.000001f;
+        const float E = ulen * (a.slack[h] + 1.01f * D::eps() + 9.5367e-7f);
+        const float margin2 = 4.f * E + ulen * 7.6294e-6f + 2.4e-7f;
+        float m2 = -INFINITY;
+        int cnt = 0;
+        for (int s = 0; s < S; s++) {
+            const float4 q = *reinterpret_cast<const float4 *>(sec + 4 * s);
+            float v[4];
+            rotate_conj(us, q.x, q.y, q.z, q.w, v);
+            const float b2 = best2_of(v);
+            m2 = fmaxf(m2, b2);
+            if (b2 >= m2 - margin2) {
+                if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
+                cnt++;
+            }
+        }
+        if (search) {
+            if (cnt > kSCap) brute = true;
+            const float thr2 = m2 - margin2;
+            int kcnt = 0;
+            if (!brute) {
+                for (int i = 0; i < cnt; i++) {
+                    const int s = slist[i][tid];
+                    const float4 q = *reinterpret_cast<const float4 *>(sec + 4 * s);
+                    float v[4];
+                    rotate_conj(us, q.x, q.y, q.z, q.w, v);
+                    if (best2_of(v) < thr2) continue;  // entered while the running maximum was lower
+#pragma unroll
+                    for (int p = 0; p < 24; p++) {
+                        if (exact2_of(v, p) >= thr2) {
+                            if (kcnt < kKCap) klist[kcnt][tid] = (uint16_t)(p * S + s);
+                            kcnt++;
+                        }
+                    }
+                }
+                if (kcnt > kKCap) brute = true;
+            }
+            if (!brute) {
+                float bs = -INFINITY;
+                int bk = 0x7fffffff;
+                for (int i = 0; i < kcnt; i++) {
+                    const int k = klist[i][tid];
+                    const float sc = ref_score<D>(u, jh + (size_t)k * 4);
+                    if (sc > bs || (sc == bs && k < bk)) { bs = sc; bk = k; }
+                }
+                idx = bk;
+            }
+        }
+        if (brute) idx = brute_argmax<D>(u, jh, K);
+        if (a.stats && active) {
+            if (brute) atomicAdd(a.stats, 1);
+            if (search && !brute) atomicAdd(a.stats + 1, cnt);
+        }
+    }
+
+    // ---- per-token scale and radius code ----
+    float rm = -INFINITY;
+    bool rm_nan = false;
+    {
+        const int base = tok_local * n;
+        for (int i = 0; i < n; i++) {
+            float o = (base + i < kQThreads) ? radius_sh[base + i] : 0.f;
+            if (is_nan(o)) rm_nan = true;
+            else if (o > rm) rm = o;
+        }
+    }
+    rm = clamp_min_d<D>(rm_nan ? NAN : rm, 1e-8f);
+    const float qmaxf = (float)a.qmax;
+    const float scale = D::rnd(rm / qmaxf);
+    float qf = rintf(D::rnd(r / scale));
+    if (!is_nan(qf)) qf = fminf(fmaxf(qf, 0.f), qmaxf);
+    const int rq = is_nan(qf) ? 0 : (int)qf;
+
+    bool flagged = false;
+    if (a.thr) flagged = nrm > D::load((const ST *)a.thr + h);
+
+    if (active) {
+        const size_t o = (((size_t)b * a.H + h) * a.T + t) * n + c;
+        if (a.idx_out) a.idx_out[o] = idx;
+        if (a.rq_out) a.rq_out[o] = rq;
+        if (a.mask_out) a.mask_out[o] = flagged ? 1 : 0;
+        if (a.rmax_out && c == 0) D::store((ST *)a.rmax_out + o / n, rm);
+        if (a.dense_out) {
+            ST *dst = (ST *)a.dense_out + o * 4;
+            if (flagged) {
+                const ST *xp = (const ST *)a.x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst + c * 4;
+                for (int j = 0; j < 4; j++) dst[j] = xp[j];
+            } else {
+                const float rqs = D::rnd(qf * scale);
+                const ST *row = jh + (size_t)idx * 4;
+                for (int j = 0; j < 4; j++) D::store(dst + j, D::rnd(rqs * D::load(row + j)));
+            }
+        }
+    }
+
+    // ---- packed rows ----
+    if (a.main_plane || a.flag_plane || a.scale_plane) {
+        code_sh[tid] = (uint32_t)idx | ((uint32_t)rq << a.idx_bits);
+        mask_sh[tid] = flagged ? 1u : 0u;
+        __syncthreads();
+        if (active) {
+            const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
+            if (row < 0 || row >= a.t_cap) return;  // a bad pos[] must not write outside the plane
+            const size_t prow = ((size_t)b * a.H + h) * a.t_cap + row;
+            const uint32_t *codes = code_sh + tok_local * n;
+            if (a.main_plane) {
+                const int rb = (n * a.main_bits + 7) >> 3;
+                uint8_t *dst = a.main_plane + prow * rb;
+                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.main_bits, 0, byte);
+            }
+            if (a.aux_plane && a.aux_bits) {
+                const int rb = (n * a.aux_bits + 7) >> 3;
+                uint8_t *dst = a.aux_plane + prow * rb;
+                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.aux_bits, a.main_bits, byte);
+            }
+            if (a.flag_plane) {
+                const int rb = (n + 7) >> 3;
+                uint8_t *dst = a.flag_plane + prow * rb;
+                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(mask_sh + tok_local * n, n, 1, 0, byte);
+            }
+            if (a.scale_plane && c == 0) D::store((ST *)a.scale_plane + prow, rm);
+        }
+    }
+}
+
+template <class D>
+static int launch_quantize(const QParams &p, int algo, hipStream_t st) {
+    dim3 grid((p.T + p.tokens_per_block - 1) / p.tokens_per_block, p.B * p.H), block(kQThreads);
+    size_t shmem = (size_t)p.S * 4 * sizeof(float);
+    if (algo == 1) hipLaunchKernelGGL((quantize_kernel<D, 1>), grid, block, shmem, st, p);
+    else hipLaunchKernelGGL((quantize_kernel<D, 0>), grid, block, shmem, st, p);
+    return hip_status(hipGetLastError());
+}
+
+}  // namespace hqmq
+
+using namespace hqmq;
+
+extern "C" int hqmq_layout_bits(int S, int radius_bits, int *idx_bits, int *main_bits, int *aux_bits) {
+    return layout_bits(S, radius_bits, idx_bits, main_bits, aux_bits);
+}
+
+extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
+    if (!a || !a->x || !a->joint) return HQMQ_ERR_NULL;
+    if (a->algo == 0 && !a->slack) return HQMQ_ERR_NULL;
+    if (a->B < 1 || a->H < 1 || a->T < 0 || a->n_chunks < 1 || a->n_chunks > kQThreads) return HQMQ_ERR_SHAPE;
+    if ((int64_t)a->B * a->H > 65535) return HQMQ_ERR_SHAPE;
+    if (a->T == 0) return HQMQ_OK;
+    int ib, mb, ab;
+    int rc = layout_bits(a->secondary_size, a->radius_bits, &ib, &mb, &ab);
+    if (rc) return rc;
+    if (24 * a->secondary_size > 65535) return HQMQ_ERR_SHAPE;  // candidate lists hold 16-bit indices
+    const bool packed = a->main_plane || a->aux_plane || a->flag_plane || a->scale_plane;
+    if (packed) {
+        if (a->main_bits != mb || a->aux_bits != ab) return HQMQ_ERR_LAYOUT;
+        if (ab && a->main_plane && !a->aux_plane) return HQMQ_ERR_NULL;
+        if (a->t_cap < 1 || a->t_off < 0) return HQMQ_ERR_SHAPE;
+        if (!a->pos && (int64_t)a->t_off + a->T > a->t_cap) return HQMQ_ERR_SHAPE;
+        if (a->flag_plane && !a->thr) return HQMQ_ERR_NULL;
+    }
+    QParams p;
+    p.x = a->x; p.xsb = a->x_stride_b; p.xsh = a->x_stride_h; p.xst = a->x_stride_t;
+    p.B = a->B; p.H = a->H; p.T = a->T; p.n = a->n_chunks;
+    p.joint = a->joint; p.slack = a->slack; p.S = a->secondary_size; p.qmax = (1 << a->radius_bits) - 1;
+    p.idx_out = a->idx_out; p.rq_out = a->rq_out; p.rmax_out = a->rmax_out; p.dense_out = a->dense_out;
+    p.thr = a->thr; p.mask_out = a->mask_out;
+    p.main_plane = a->main_plane; p.aux_plane = a->aux_plane; p.flag_plane = a->flag_plane;
+    p.scale_plane = a->scale_plane; p.t_cap = a->t_cap; p.t_off = a->t_off; p.pos = a->pos;
+    p.idx_bits = ib; p.main_bits = mb; p.aux_bits = ab;
+    p.tokens_per_block = kQThreads / a->n_chunks;
+    p.stats = a->stats;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a->dtype) {
+        case HQMQ_F32: return launch_quantize<F32>(p, a->algo, st);
+        case HQMQ_F16: return launch_quantize<F16>(p, a->algo, st);
+        case HQMQ_BF16: return launch_quantize<BF16>(p, a->algo, st);
+        default: return HQMQ_ERR_DTYPE;
+    }
+}

@@ -1,0 +1,179 @@
+/* hqmq_amd.h — C ABI of libhqmq_amd.so: the HQMQ KV-cache path on MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, explicit sizes and a HIP stream
+ * (void*, NULL = the null stream), enqueues its kernels on that stream and
+ * returns without synchronising.  The library allocates nothing: outputs and
+ * scratch are caller-owned device buffers.  Return value: 0 = ok, negative =
+ * argument error (hqmq_status_string explains), positive = hipError_t.
+ *
+ * The reference is pure Python (PyTorch + Triton) and has no FFI; each entry
+ * point names the reference function whose work it replaces.  A Python caller
+ * binds these with ctypes (see hqmq_amd/_lib.py).
+ *
+ * Element types: HQMQ_F32 / HQMQ_F16 / HQMQ_BF16 name the dtype D of the K/V
+ * tensor.  All arithmetic that decides an integer (codeword index, radius
+ * code, Med3x mask) reproduces torch's CPU rounding in D.
+ *
+ * Packed cache layout (one "plane set" per tensor K or V of one layer), all
+ * planes contiguous [B][H][t_cap][row]:
+ *   code      = idx | rq << idx_bits,  idx_bits = ceil(log2(24*S)), rq < 2^radius_bits
+ *   main row  = little-endian bit stream of the low main_bits of each of the n codes
+ *   aux row   = bit stream of the remaining aux_bits (absent when aux_bits == 0)
+ *   scale     = per-token r_max in D
+ *   flags row = 1 bit per chunk (Med3x outlier), n/8 bytes            (optional)
+ *   sideband  = [B][H][sb_cap][4] in D: the flagged chunks verbatim, in
+ *               (token, chunk) order; sb_tile_off[B][H][t_cap/16] = number of
+ *               flagged chunks before token 16*i; sb_count[B][H] = total.
+ *   s24_r3 -> 12+1 bits (48+4 B/token at d_h=128), s96_r4 -> 16+0 (64 B),
+ *   s192_r6 -> 16+3 (64+12 B).
+ */
+#ifndef HQMQ_AMD_H
+#define HQMQ_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { HQMQ_F32 = 0, HQMQ_F16 = 1, HQMQ_BF16 = 2 };
+
+enum {
+    HQMQ_OK = 0,
+    HQMQ_ERR_NULL = -1,      /* a required pointer is NULL */
+    HQMQ_ERR_SHAPE = -2,     /* a size is out of the supported range */
+    HQMQ_ERR_DTYPE = -3,     /* unknown or unsupported dtype */
+    HQMQ_ERR_LAYOUT = -4,    /* bit widths inconsistent with the layout rules */
+    HQMQ_ERR_WORKSPACE = -5, /* workspace too small */
+    HQMQ_ERR_ALIGN = -6      /* a pointer or stride is not aligned as required */
+};
+
+int hqmq_version(void);                    /* 0xMMmmpp */
+const char *hqmq_status_string(int status);
+
+/* Bit widths of the packed layout for a codebook of 24*S codewords and
+ * radius_bits radius bits.  Any output pointer may be NULL. */
+int hqmq_layout_bits(int secondary_size, int radius_bits, int *idx_bits, int *main_bits, int *aux_bits);
+
+/* Joint codebook q_p*q_s in D with the reference's op-by-op rounding, k = p*S + s.
+ * Replaces HQMQQuantizer._get_codebook (src/quantizers/hqmq.py:119-143).
+ *   raw    [H][S][4] fp32, unnormalised secondary parameters of one (layer, K|V)
+ *   joint  [H][24*S][4] in D (out)
+ *   slack  [H] fp32 (out): max_k || joint[k] - exact(q_p*q_s) ||_2, the bound the
+ *          quantize kernel's candidate filter needs */
+int hqmq_build_joint(const float *raw, int H, int S, int dtype, void *joint, float *slack, void *stream);
+
+/* Quantize (and optionally pack) x[B][H][T][4n].
+ * Replaces HQMQQuantizer._qdq (src/quantizers/hqmq.py:145-216, unit magnitude,
+ * linear radius) and, when thr != NULL, the mask/merge half of
+ * OutlierAwareHQMQQuantizer._qdq (src/quantizers/outlier_aware.py:72,86).
+ * Any output may be NULL. */
+typedef struct hqmq_quantize_args {
+    const void *x;            /* D, last dim contiguous */
+    int64_t x_stride_b, x_stride_h, x_stride_t; /* in elements */
+    int dtype;
+    int B, H, T, n_chunks;
+    const void *joint;        /* [H][24*S][4] D */
+    const float *slack;       /* [H] from hqmq_build_joint */
+    int secondary_size, radius_bits;
+    int algo;                 /* 0 = closed-form filter + exact re-score, 1 = brute force */
+    /* unpacked outputs, contiguous [B][H][T][n] / [B][H][T] / [B][H][T][4n] */
+    int32_t *idx_out, *rq_out;
+    void *rmax_out;           /* D */
+    void *dense_out;          /* D: the reference's fake-quant tensor (outlier chunks restored if thr) */
+    /* Med3x: per-head threshold in D; mask = ||chunk|| > thr */
+    const void *thr;          /* [H] D or NULL */
+    uint8_t *mask_out;        /* [B][H][T][n] bytes or NULL */
+    /* packed outputs: row (pos ? pos[b] : 0) + t_off + t of each [B][H][t_cap] plane */
+    uint8_t *main_plane, *aux_plane, *flag_plane;
+    void *scale_plane;        /* D */
+    int64_t t_cap;
+    int t_off;
+    const int32_t *pos;       /* [B] or NULL */
+    int main_bits, aux_bits;
+    int32_t *stats;           /* [2] or NULL, accumulated: lanes that scored all rows; secondaries kept by the filter */
+} hqmq_quantize_args;
+int hqmq_quantize(const hqmq_quantize_args *a, void *stream);
+
+/* Med3x statistics: per-head median of the chunk norms of one call and the
+ * threshold RNE_D(median * mult).  Replaces the torch.quantile half of
+ * OutlierAwareHQMQQuantizer._qdq (src/quantizers/outlier_aware.py:60-69).
+ *   workspace  hqmq_med3x_workspace_bytes(H, dtype) bytes, any content
+ *   median     [H] fp32 (out);  thr [H] D (out);  n_out [H] int32 (out, may be NULL):
+ *              number of chunks with norm > thr */
+int64_t hqmq_med3x_workspace_bytes(int H, int dtype);
+int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype,
+                         int B, int H, int T, int n_chunks, float mult, void *workspace, int64_t workspace_bytes,
+                         float *median, void *thr, int32_t *n_out, void *stream);
+
+/* Compact the flagged chunks of rows [row0, row0+T) into the sideband.
+ * No counterpart in the reference (its wrapper keeps a dense tensor).
+ * Rows must be appended in order; row0 = (pos ? pos[b] : 0) + t_off. */
+int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype,
+                         int B, int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
+                         const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off, int32_t *sb_count,
+                         int32_t *overflow, void *stream);
+
+/* Dense decode of unpacked codes: out = joint[h, idx] * ((rq * rs) / qmax) in D.
+ * Replaces hqmq_decode_triton (src/quantizers/hqmq_kernel.py:102-132) with the
+ * rounding of _decode_kv_torch (src/quantizers/hqmq_attention.py:39-65).
+ * Strides in elements; idx/rq last dim contiguous; out contiguous [B][H][T][4n]. */
+int hqmq_dequant(const int32_t *idx, int64_t idx_sb, int64_t idx_sh, int64_t idx_st,
+                 const int32_t *rq, int64_t rq_sb, int64_t rq_sh, int64_t rq_st,
+                 const void *rs, int64_t rs_sb, int64_t rs_sh, int64_t rs_st,
+                 const void *joint, int64_t joint_sh, int K, int dtype, int B, int H, int T, int n_chunks,
+                 int qmax, void *out, void *stream);
+
+/* Pack unpacked codes into main/aux/scale rows (for callers that hold the
+ * reference's int32 representation).  No counterpart in the reference. */
+int hqmq_pack_codes(const int32_t *idx, int64_t idx_sb, int64_t idx_sh, int64_t idx_st,
+                    const int32_t *rq, int64_t rq_sb, int64_t rq_sh, int64_t rq_st,
+                    int B, int H, int T, int n_chunks, int idx_bits, int main_bits, int aux_bits,
+                    uint8_t *main_plane, uint8_t *aux_plane, int64_t t_cap, void *stream);
+
+/* One packed tensor (K or V) as the attention and dense-decode kernels read it. */
+typedef struct hqmq_packed {
+    const uint8_t *main_plane, *aux_plane, *flag_plane; /* aux/flag may be NULL */
+    const void *scale_plane;  /* D, or any float dtype given by scale_dtype */
+    int64_t scale_sb, scale_sh, scale_st; /* element strides of scale_plane (contiguous: H*t_cap, t_cap, 1) */
+    const void *sideband;     /* NULL when flag_plane is NULL */
+    const int32_t *sb_tile_off;
+    int64_t sb_cap;
+    const void *joint;        /* [H][K][4] D */
+    int64_t joint_sh;         /* element stride between heads */
+    int K;                    /* codewords in joint */
+} hqmq_packed;
+
+/* Dense decode of a packed cache (outlier chunks substituted from the sideband). */
+int hqmq_dequant_packed(const hqmq_packed *p, int dtype, int B, int H, int T, int n_chunks, int64_t t_cap,
+                        int idx_bits, int main_bits, int aux_bits, int qmax, void *out, void *stream);
+
+/* Fused attention over the packed cache: decode (T_q = 1) and chunked prefill.
+ * Replaces fused_hqmq_attention_triton (src/quantizers/hqmq_attention.py:425-518)
+ * with the semantics of fused_hqmq_attention_torch (:68-101).
+ * Query row i of sequence b sees key j iff j < kv_len[b] (T_kv when kv_len is
+ * NULL) and (not causal or j <= i + causal_offset); causal_offset = 0 is the
+ * reference's top-left alignment.
+ *   workspace   hqmq_attn_workspace_bytes(...) bytes of scratch for split-KV partials */
+typedef struct hqmq_attn_args {
+    const void *Q; void *O;   /* D, [B][H_q][T_q][d_h]; strides in elements, last dim contiguous */
+    int64_t q_sb, q_sh, q_st, o_sb, o_sh, o_st;
+    hqmq_packed K, V;
+    int dtype;
+    int B, H_q, H_kv, T_q, T_kv, n_chunks;
+    int64_t t_cap;
+    int idx_bits, main_bits, aux_bits, qmax;
+    const int32_t *kv_len;    /* [B] or NULL */
+    int causal; int64_t causal_offset;
+    float softmax_scale;
+    int n_splits;             /* 0 = choose */
+    void *workspace; int64_t workspace_bytes;
+} hqmq_attn_args;
+int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
+int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv);
+int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HQMQ_AMD_H */
