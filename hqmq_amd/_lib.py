@@ -62,7 +62,7 @@ class AttnArgs(C.Structure):
 
 EXPORTS = [
     "hqmq_version", "hqmq_status_string", "hqmq_layout_bits", "hqmq_build_joint", "hqmq_quantize",
-    "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_compact", "hqmq_dequant",
+    "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",
     "hqmq_pack_codes", "hqmq_dequant_packed", "hqmq_attn_workspace_bytes", "hqmq_attn_pick_splits",
     "hqmq_attn_fwd",
 ]
@@ -82,7 +82,6 @@ def lib():
         L.hqmq_status_string.restype = C.c_char_p
         L.hqmq_status_string.argtypes = [C.c_int]
         for name in ("hqmq_med3x_workspace_bytes", "hqmq_attn_workspace_bytes"):
-            if not hasattr(L, name): continue  # TEMP
             getattr(L, name).restype = i64
         _lib = L
     return _lib

@@ -1,0 +1,371 @@
+// Med3x outlier statistics and sideband compaction.
+//
+// hqmq_med3x_threshold follows the torch.quantile half of
+// OutlierAwareHQMQQuantizer._qdq (src/quantizers/outlier_aware.py:60-69 of the
+// reference): per head, the median over every chunk norm of the call (fp32
+// interpolation between the two middle order statistics), times the
+// multiplier, rounded to D.  The order statistics come from an exact radix
+// select: chunk norms are non-negative, so their bit patterns sort like the
+// values; 16-bit dtypes need one 32768-bin histogram per head, fp32 a second
+// pass over the low 16 bits of the bin(s) holding the two ranks.
+//
+// hqmq_outlier_compact has no counterpart in the reference: it copies the
+// flagged chunks into the fp16/bf16/fp32 sideband in (token, chunk) order.
+//
+// Compiled with -ffp-contract=off.
+#include "common.h"
+
+namespace hqmq {
+
+constexpr int kBins1 = 32768;
+constexpr int kBins2 = 65536;
+constexpr int kState = 16;  // ints per head
+
+// workspace (uint32 units): hist1[H][kBins1] | state[H][kState] | (fp32 only) hist2[H][2][kBins2]
+// state: 0 nan count, 1 key_lo, 2 key_hi, 3 rank_lo within bin, 4 rank_hi within bin
+__host__ __device__ inline int64_t ws_words(int H, bool f32) {
+    return (int64_t)H * (kBins1 + kState) + (f32 ? (int64_t)H * 2 * kBins2 : 0);
+}
+
+__global__ void fill_zero_kernel(uint32_t *p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+template <class D>
+__device__ __forceinline__ float chunk_norm(const typename D::storage *xp) {
+    return D::rnd(norm4(D::load(xp), D::load(xp + 1), D::load(xp + 2), D::load(xp + 3)));
+}
+
+template <class D>
+__device__ __forceinline__ uint32_t norm_bits(float nrm) {
+    if (D::code == HQMQ_F32) return __float_as_uint(nrm);
+    if (D::code == HQMQ_F16) return (uint32_t)__half_as_ushort(__float2half_rn(nrm)) << 16;
+    return __float_as_uint(nrm);  // bf16 value: low 16 bits are zero
+}
+
+// LEVEL 0: histogram of the top 16 bits. LEVEL 1 (fp32): low 16 bits of norms whose top bits match a selected bin.
+template <class D, int LEVEL>
+__global__ void med_hist_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int B, int H, int T, int n,
+                                uint32_t *ws) {
+    const int h = blockIdx.y;
+    uint32_t *hist1 = ws + (size_t)h * kBins1;
+    uint32_t *state = ws + (size_t)H * kBins1 + (size_t)h * kState;
+    uint32_t *hist2 = ws + (size_t)H * (kBins1 + kState) + (size_t)h * 2 * kBins2;
+    const int64_t per_head = (int64_t)B * T * n;
+    uint32_t key_lo = 0, key_hi = 0;
+    if (LEVEL == 1) { key_lo = state[1]; key_hi = state[2]; }
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < per_head; g += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(g % n);
+        const int64_t bt = g / n;
+        const int t = (int)(bt % T), b = (int)(bt / T);
+        const float nrm = chunk_norm<D>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4);
+        if (is_nan(nrm)) {
+            if (LEVEL == 0) atomicAdd(&state[0], 1u);
+            continue;
+        }
+        const uint32_t bits = norm_bits<D>(nrm);
+        if (LEVEL == 0) atomicAdd(&hist1[bits >> 16], 1u);
+        else {
+            if ((bits >> 16) == key_lo) atomicAdd(&hist2[bits & 0xffffu], 1u);
+            if ((bits >> 16) == key_hi && key_hi != key_lo) atomicAdd(&hist2[kBins2 + (bits & 0xffffu)], 1u);
+        }
+    }
+}
+
+// Finds the bins holding 0-based ranks r_lo <= r_hi in a histogram of `bins` counters.
+// One block of 1024 threads; results through shared memory.
+__device__ void select_two(const uint32_t *hist, int bins, int64_t r_lo, int64_t r_hi, uint32_t *key_lo, uint32_t *key_hi,
+                           int64_t *in_lo, int64_t *in_hi) {
+    __shared__ unsigned long long part[1024];
+    __shared__ uint32_t res[2];
+    __shared__ long long resr[2];
+    const int per = bins / 1024;
+    unsigned long long s = 0;
+    for (int i = 0; i < per; i++) s += hist[threadIdx.x * per + i];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long run = 0;
+        int which = 0;
+        const int64_t want[2] = {r_lo, r_hi};
+        for (int i = 0; i < 1024 && which < 2; i++) {
+            while (which < 2 && (unsigned long long)want[which] < run + part[i]) {
+                unsigned long long r2 = run;
+                for (int j = 0; j < per; j++) {
+                    const uint32_t cnt = hist[i * per + j];
+                    if ((unsigned long long)want[which] < r2 + cnt) {
+                        res[which] = (uint32_t)(i * per + j);
+                        resr[which] = (long long)((unsigned long long)want[which] - r2);
+                        break;
+                    }
+                    r2 += cnt;
+                }
+                which++;
+            }
+            run += part[i];
+        }
+    }
+    __syncthreads();
+    *key_lo = res[0]; *key_hi = res[1];
+    *in_lo = resr[0]; *in_hi = resr[1];
+    __syncthreads();
+}
+
+template <class D>
+__device__ __forceinline__ void finish_threshold(float a, float b, bool same, float mult, int h, float *median,
+                                                 typename D::storage *thr) {
+    float med;
+    if (same) med = a;
+    else {
+        const float d = b - a;
+        const float e = d * 0.5f;
+        med = b - e;
+    }
+    median[h] = med;
+    const float t32 = med * mult;
+    D::store(thr + h, D::rnd(t32));
+}
+
+template <class D>
+__global__ __launch_bounds__(1024) void med_select1_kernel(uint32_t *ws, int H, int64_t per_head, float mult, float *median,
+                                                           typename D::storage *thr, int32_t *n_out) {
+    const int h = blockIdx.x;
+    const uint32_t *hist1 = ws + (size_t)h * kBins1;
+    uint32_t *state = ws + (size_t)H * kBins1 + (size_t)h * kState;
+    if (state[0] > 0) {  // a NaN norm makes the quantile NaN, the mask empty
+        if (threadIdx.x == 0) {
+            median[h] = NAN;
+            D::store(thr + h, NAN);
+            if (n_out) n_out[h] = 0;
+            state[1] = 0xffffffffu; state[2] = 0xffffffffu;
+        }
+        return;
+    }
+    uint32_t klo, khi;
+    int64_t ilo, ihi;
+    select_two(hist1, kBins1, (per_head - 1) / 2, per_head / 2, &klo, &khi, &ilo, &ihi);
+    if (D::code == HQMQ_F32) {
+        if (threadIdx.x == 0) { state[1] = klo; state[2] = khi; state[3] = (uint32_t)ilo; state[4] = (uint32_t)ihi; }
+        return;
+    }
+    __shared__ float thr_sh;
+    if (threadIdx.x == 0) {
+        const float a = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)klo)) : __uint_as_float(klo << 16);
+        const float b = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)khi)) : __uint_as_float(khi << 16);
+        finish_threshold<D>(a, b, (per_head - 1) / 2 == per_head / 2, mult, h, median, thr);
+        thr_sh = D::load(thr + h);
+    }
+    __syncthreads();
+    if (n_out) {  // chunks with norm > thr: bins above the threshold's own bin
+        __shared__ unsigned long long cnt_sh;
+        if (threadIdx.x == 0) cnt_sh = 0;
+        __syncthreads();
+        const float tv = thr_sh;
+        unsigned long long s = 0;
+        for (int k = threadIdx.x; k < kBins1; k += blockDim.x) {
+            const float v = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)k)) : __uint_as_float((uint32_t)k << 16);
+            if (v > tv) s += hist1[k];
+        }
+        atomicAdd(&cnt_sh, s);
+        __syncthreads();
+        if (threadIdx.x == 0) n_out[h] = (int32_t)cnt_sh;
+    }
+}
+
+__global__ __launch_bounds__(1024) void med_select2_kernel(uint32_t *ws, int H, int64_t per_head, float mult, float *median,
+                                                           float *thr) {
+    const int h = blockIdx.x;
+    uint32_t *state = ws + (size_t)H * kBins1 + (size_t)h * kState;
+    const uint32_t *hist2 = ws + (size_t)H * (kBins1 + kState) + (size_t)h * 2 * kBins2;
+    if (state[0] > 0) return;
+    const uint32_t klo = state[1], khi = state[2];
+    uint32_t l0, l1, d0, d1;
+    int64_t i0, i1;
+    if (klo == khi) {
+        select_two(hist2, kBins2, state[3], state[4], &l0, &l1, &i0, &i1);
+    } else {
+        select_two(hist2, kBins2, state[3], state[3], &l0, &d0, &i0, &i1);
+        select_two(hist2 + kBins2, kBins2, state[4], state[4], &l1, &d1, &i0, &i1);
+    }
+    if (threadIdx.x == 0) {
+        const float a = __uint_as_float((klo << 16) | l0), b = __uint_as_float((khi << 16) | l1);
+        finish_threshold<F32>(a, b, (per_head - 1) / 2 == per_head / 2, mult, h, median, thr);
+    }
+}
+
+__global__ void count_gt_kernel(const float *x, int64_t xsb, int64_t xsh, int64_t xst, int B, int T, int n, const float *thr,
+                                int32_t *n_out) {
+    const int h = blockIdx.y;
+    const float tv = thr[h];
+    const int64_t per_head = (int64_t)B * T * n;
+    int cnt = 0;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < per_head; g += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(g % n);
+        const int64_t bt = g / n;
+        const int t = (int)(bt % T), b = (int)(bt / T);
+        if (chunk_norm<F32>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4) > tv) cnt++;
+    }
+    if (cnt) atomicAdd(&n_out[h], cnt);
+}
+
+// One block per (b, h): walks the T new rows in order, 1024 rows per step.
+template <class D>
+__global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H,
+                                                        int T, int n, const uint8_t *flag_plane, int64_t t_cap, int t_off,
+                                                        const int32_t *pos, typename D::storage *sideband, int64_t sb_cap,
+                                                        int32_t *sb_tile_off, int32_t *sb_count, int32_t *overflow) {
+    using ST = typename D::storage;
+    __shared__ int scan[1024];
+    __shared__ int base_sh;
+    const int bh = blockIdx.x, b = bh / H, h = bh - b * H;
+    const int frb = (n + 7) >> 3;
+    const int64_t row0 = (pos ? pos[b] : 0) + t_off;
+    const int64_t tiles = (t_cap + kTile - 1) / kTile;
+    if (threadIdx.x == 0) base_sh = sb_count[bh];
+    __syncthreads();
+    for (int t0 = 0; t0 < T; t0 += 1024) {
+        const int t = t0 + threadIdx.x;
+        const int64_t row = row0 + t;
+        const bool live = t < T && row < t_cap;
+        int cnt = 0;
+        const uint8_t *fr = flag_plane + ((size_t)bh * t_cap + (live ? row : 0)) * frb;
+        if (live)
+            for (int by = 0; by < frb; by++) cnt += __popc((uint32_t)fr[by]);
+        scan[threadIdx.x] = cnt;
+        __syncthreads();
+        for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scan
+            int v = (int)threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
+            __syncthreads();
+            scan[threadIdx.x] += v;
+            __syncthreads();
+        }
+        const int base = base_sh;
+        const int before = base + scan[threadIdx.x] - cnt;
+        if (live) {
+            if ((row & (kTile - 1)) == 0) sb_tile_off[(size_t)bh * tiles + (row >> 4)] = before;
+            int k = before;
+            const ST *xr = x + b * xsb + h * xsh + (int64_t)t * xst;
+            for (int c = 0; c < n && cnt; c++) {
+                if ((fr[c >> 3] >> (c & 7)) & 1) {
+                    if (k < sb_cap) {
+                        ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
+                        for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
+                    } else *overflow = 1;
+                    k++;
+                }
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) base_sh = base + scan[1023];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) sb_count[bh] = base_sh;
+}
+
+}  // namespace hqmq
+
+using namespace hqmq;
+
+extern "C" int64_t hqmq_med3x_workspace_bytes(int H, int dtype) {
+    if (H < 1) return 0;
+    return ws_words(H, dtype == HQMQ_F32) * 4;
+}
+
+template <class D>
+static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B, int H, int T, int n, float mult, uint32_t *ws,
+                     float *median, void *thr, int32_t *n_out, hipStream_t st) {
+    using ST = typename D::storage;
+    const bool f32 = D::code == HQMQ_F32;
+    const int64_t words = ws_words(H, f32);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, ws, words);
+    const int64_t per_head = (int64_t)B * T * n;
+    int gx = (int)((per_head + 255) / 256);
+    if (gx > 2048) gx = 2048;
+    hipLaunchKernelGGL((med_hist_kernel<D, 0>), dim3(gx, H), dim3(256), 0, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
+    hipLaunchKernelGGL(med_select1_kernel<D>, dim3(H), dim3(1024), 0, st, ws, H, per_head, mult, median, (ST *)thr, n_out);
+    if (f32) {
+        hipLaunchKernelGGL((med_hist_kernel<D, 1>), dim3(gx, H), dim3(256), 0, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
+        hipLaunchKernelGGL(med_select2_kernel, dim3(H), dim3(1024), 0, st, ws, H, per_head, mult, median, (float *)thr);
+        if (n_out) {
+            hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, st, (uint32_t *)n_out, (int64_t)H);
+            hipLaunchKernelGGL(count_gt_kernel, dim3(gx, H), dim3(256), 0, st, (const float *)x, xsb, xsh, xst, B, T, n,
+                               (const float *)thr, n_out);
+        }
+    }
+    return hip_status(hipGetLastError());
+}
+
+extern "C" int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
+                                    int H, int T, int n_chunks, float mult, void *workspace, int64_t workspace_bytes,
+                                    float *median, void *thr, int32_t *n_out, void *stream) {
+    if (!x || !workspace || !median || !thr) return HQMQ_ERR_NULL;
+    if (B < 1 || H < 1 || H > 65535 || T < 1 || n_chunks < 1) return HQMQ_ERR_SHAPE;
+    if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
+    if (workspace_bytes < hqmq_med3x_workspace_bytes(H, dtype)) return HQMQ_ERR_WORKSPACE;
+    if (((uintptr_t)workspace & 3) != 0) return HQMQ_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *ws = (uint32_t *)workspace;
+    switch (dtype) {
+        case HQMQ_F32: return run_med3x<F32>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
+        case HQMQ_F16: return run_med3x<F16>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
+        default: return run_med3x<BF16>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
+    }
+}
+
+extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
+                                    int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
+                                    const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off,
+                                    int32_t *sb_count, int32_t *overflow, void *stream) {
+    if (!x || !flag_plane || !sideband || !sb_tile_off || !sb_count || !overflow) return HQMQ_ERR_NULL;
+    if (B < 1 || H < 1 || T < 0 || n_chunks < 1 || t_cap < 1 || sb_cap < 1 || t_off < 0) return HQMQ_ERR_SHAPE;
+    if (T == 0) return HQMQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(B * H), block(1024);
+#define LAUNCH(DT, ST)                                                                                                      \
+    hipLaunchKernelGGL(compact_kernel<DT>, grid, block, 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T, n_chunks, \
+                       flag_plane, t_cap, t_off, pos, (ST *)sideband, sb_cap, sb_tile_off, sb_count, overflow)
+    switch (dtype) {
+        case HQMQ_F32: LAUNCH(F32, float); break;
+        case HQMQ_F16: LAUNCH(F16, uint16_t); break;
+        case HQMQ_BF16: LAUNCH(BF16, uint16_t); break;
+        default: return HQMQ_ERR_DTYPE;
+    }
+#undef LAUNCH
+    return hip_status(hipGetLastError());
+}
+
+namespace hqmq {
+template <class D>
+__global__ void outlier_mask_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int B, int H, int T, int n,
+                                    const typename D::storage *thr, uint8_t *mask) {
+    const int64_t total = (int64_t)B * H * T * n;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(g % n);
+        const int64_t row = g / n;
+        const int t = (int)(row % T), h = (int)((row / T) % H), b = (int)(row / ((int64_t)T * H));
+        mask[g] = chunk_norm<D>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4) > D::load(thr + h) ? 1 : 0;
+    }
+}
+}  // namespace hqmq
+
+extern "C" int hqmq_outlier_mask(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
+                                 int H, int T, int n_chunks, const void *thr, uint8_t *mask, void *stream) {
+    if (!x || !thr || !mask) return HQMQ_ERR_NULL;
+    if (B < 1 || H < 1 || T < 0 || n_chunks < 1) return HQMQ_ERR_SHAPE;
+    if (T == 0) return HQMQ_OK;
+    const int64_t total = (int64_t)B * H * T * n_chunks;
+    int64_t g = (total + 255) / 256;
+    if (g > (1 << 20)) g = 1 << 20;
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(DT, ST)                                                                                                      \
+    hipLaunchKernelGGL(outlier_mask_kernel<DT>, dim3((unsigned)g), dim3(256), 0, st, (const ST *)x, x_stride_b, x_stride_h, \
+                       x_stride_t, B, H, T, n_chunks, (const ST *)thr, mask)
+    switch (dtype) {
+        case HQMQ_F32: LAUNCH(F32, float); break;
+        case HQMQ_F16: LAUNCH(F16, uint16_t); break;
+        case HQMQ_BF16: LAUNCH(BF16, uint16_t); break;
+        default: return HQMQ_ERR_DTYPE;
+    }
+#undef LAUNCH
+    return hip_status(hipGetLastError());
+}

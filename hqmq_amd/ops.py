@@ -102,3 +102,165 @@ def quantize(x: torch.Tensor, joint: torch.Tensor, slack: Optional[torch.Tensor]
     if "mask8" in out:
         out["mask"] = out.pop("mask8").bool()
     return out
+
+
+_WS = {}
+
+
+def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
+    """A cached scratch buffer of at least nbytes (grown on demand, reused across calls)."""
+    key = (tag, torch.device(device))
+    buf = _WS.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        _WS[key] = buf
+    return buf
+
+
+def med3x_threshold(x: torch.Tensor, mult: float = 3.0, want_count: bool = True):
+    """Per-head (median fp32, threshold in x.dtype, #chunks above threshold int32) over the whole call."""
+    L.require_gpu(x, "x")
+    x = _strided_x(x)
+    B, H, T, d_h = x.shape
+    n = d_h // 4
+    dev = x.device
+    nbytes = int(L.lib().hqmq_med3x_workspace_bytes(C.c_int(H), C.c_int(_dt(x))))
+    ws = _workspace(nbytes, dev, "med3x")
+    med = torch.empty(H, dtype=torch.float32, device=dev)
+    thr = torch.empty(H, dtype=x.dtype, device=dev)
+    cnt = torch.zeros(H, dtype=torch.int32, device=dev) if want_count else None
+    with torch.cuda.device(dev):
+        L.check(L.lib().hqmq_med3x_threshold(
+            L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
+            C.c_int(T), C.c_int(n), C.c_float(mult), L.ptr(ws), L.i64(ws.numel()), L.ptr(med), L.ptr(thr), L.ptr(cnt),
+            L.stream_ptr(dev)), "hqmq_med3x_threshold")
+    return med, thr, cnt
+
+
+def outlier_mask(x: torch.Tensor, thr: torch.Tensor) -> torch.Tensor:
+    """Boolean (B, H, T, n) mask of chunks whose norm exceeds the per-head threshold."""
+    L.require_gpu(x, "x")
+    x = _strided_x(x)
+    B, H, T, d_h = x.shape
+    thr = thr.to(x.dtype).contiguous()
+    mask = torch.empty(B, H, T, d_h // 4, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().hqmq_outlier_mask(
+            L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
+            C.c_int(T), C.c_int(d_h // 4), L.ptr(thr), L.ptr(mask), L.stream_ptr(x.device)), "hqmq_outlier_mask")
+    return mask.bool()
+
+
+def outlier_compact(x: torch.Tensor, cache, t_off: int = 0, pos: Optional[torch.Tensor] = None) -> None:
+    """Append the flagged chunks of x (rows t_off.. of the cache) to the cache's sideband."""
+    x = _strided_x(x)
+    B, H, T, d_h = x.shape
+    dev = x.device
+    if pos is not None:
+        pos = pos.to(device=dev, dtype=torch.int32).contiguous()
+    with torch.cuda.device(dev):
+        L.check(L.lib().hqmq_outlier_compact(
+            L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
+            C.c_int(T), C.c_int(d_h // 4), L.ptr(cache.flags), L.i64(cache.t_cap), C.c_int(t_off), L.ptr(pos),
+            L.ptr(cache.sideband), L.i64(cache.sb_cap), L.ptr(cache.sb_tile_off), L.ptr(cache.sb_count),
+            L.ptr(cache.sb_overflow), L.stream_ptr(dev)), "hqmq_outlier_compact")
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    t = t if t.dtype == torch.int32 else t.to(torch.int32)
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def dequant(idx, radius_q, radius_scale, joint, r_qmax: int) -> torch.Tensor:
+    """Unpacked codes -> dense (B, H, T, 4n) in joint.dtype (rounding of the reference's torch decode)."""
+    L.require_gpu(idx, "idx")
+    idx, rq = _i32(idx), _i32(radius_q)
+    B, H, T, n = idx.shape
+    rs = radius_scale.to(joint.dtype)
+    if joint.stride(-1) != 1 or joint.stride(1) != 4:
+        joint = joint.contiguous()
+    out = torch.empty(B, H, T, 4 * n, dtype=joint.dtype, device=idx.device)
+    with torch.cuda.device(idx.device):
+        L.check(L.lib().hqmq_dequant(
+            L.ptr(idx), L.i64(idx.stride(0)), L.i64(idx.stride(1)), L.i64(idx.stride(2)),
+            L.ptr(rq), L.i64(rq.stride(0)), L.i64(rq.stride(1)), L.i64(rq.stride(2)),
+            L.ptr(rs), L.i64(rs.stride(0)), L.i64(rs.stride(1)), L.i64(rs.stride(2)),
+            L.ptr(joint), L.i64(joint.stride(0)), C.c_int(joint.shape[1]), C.c_int(_dt(joint)), C.c_int(B), C.c_int(H),
+            C.c_int(T), C.c_int(n), C.c_int(r_qmax), L.ptr(out), L.stream_ptr(idx.device)), "hqmq_dequant")
+    return out
+
+
+def pack_codes(idx, radius_q, cache, T: Optional[int] = None) -> None:
+    """Write unpacked int codes into rows [0, T) of a PackedTensor's code planes."""
+    idx, rq = _i32(idx), _i32(radius_q)
+    B, H, Ti, n = idx.shape
+    T = Ti if T is None else T
+    with torch.cuda.device(idx.device):
+        L.check(L.lib().hqmq_pack_codes(
+            L.ptr(idx), L.i64(idx.stride(0)), L.i64(idx.stride(1)), L.i64(idx.stride(2)),
+            L.ptr(rq), L.i64(rq.stride(0)), L.i64(rq.stride(1)), L.i64(rq.stride(2)),
+            C.c_int(B), C.c_int(H), C.c_int(T), C.c_int(n), C.c_int(cache.idx_bits), C.c_int(cache.main_bits),
+            C.c_int(cache.aux_bits), L.ptr(cache.main), L.ptr(cache.aux), L.i64(cache.t_cap), L.stream_ptr(idx.device)),
+            "hqmq_pack_codes")
+
+
+def dequant_packed(cache, T: Optional[int] = None, mode: int = 0) -> torch.Tensor:
+    """Packed cache -> dense (B, H, T, d_h); mode 0 = attention rounding, 1 = quantizer fake-quant rounding."""
+    T = cache.length if T is None else T
+    out = torch.empty(cache.B, cache.H, T, cache.d_head, dtype=cache.dtype, device=cache.device)
+    s = cache.c_struct()
+    with torch.cuda.device(cache.device):
+        L.check(L.lib().hqmq_dequant_packed(
+            C.byref(s), C.c_int(L.DT_CODE[cache.dtype]), C.c_int(cache.B), C.c_int(cache.H), C.c_int(T), C.c_int(cache.n),
+            L.i64(cache.t_cap), C.c_int(cache.idx_bits), C.c_int(cache.main_bits), C.c_int(cache.aux_bits),
+            C.c_int(cache.qmax), C.c_int(mode), L.ptr(out), L.stream_ptr(cache.device)), "hqmq_dequant_packed")
+    return out
+
+
+def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int) -> int:
+    return int(L.lib().hqmq_attn_pick_splits(C.c_int(B), C.c_int(H_q), C.c_int(H_kv), C.c_int(T_q), C.c_int(T_kv)))
+
+
+def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None, causal: bool = False,
+             causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each)."""
+    L.require_gpu(Q, "Q")
+    if Q.stride(-1) != 1:
+        Q = Q.contiguous()
+    B, Hq, Tq, d_h = Q.shape
+    if d_h != Kc.d_head or d_h != Vc.d_head:
+        raise AssertionError(f"d_h={d_h} != n_chunks*4={Kc.d_head}")
+    if Hq % Kc.H:
+        raise AssertionError(f"H_q={Hq} must be divisible by H_kv={Kc.H}")
+    if Q.dtype != Kc.dtype:
+        raise L.HqmqError(f"Q dtype {Q.dtype} differs from the cache dtype {Kc.dtype}")
+    dev = Q.device
+    O = out if out is not None else torch.empty_like(Q)
+    if softmax_scale is None:
+        softmax_scale = d_h ** -0.5
+    if n_splits <= 0:
+        n_splits = pick_splits(B, Hq, Kc.H, Tq, max(T_kv, 1))
+    a = L.AttnArgs()
+    a.Q, a.O = L.ptr(Q), L.ptr(O)
+    a.q_sb, a.q_sh, a.q_st = Q.stride(0), Q.stride(1), Q.stride(2)
+    a.o_sb, a.o_sh, a.o_st = O.stride(0), O.stride(1), O.stride(2)
+    a.K, a.V = Kc.c_struct(), Vc.c_struct()
+    a.dtype = L.DT_CODE[Q.dtype]
+    a.B, a.H_q, a.H_kv, a.T_q, a.T_kv, a.n_chunks = B, Hq, Kc.H, Tq, T_kv, Kc.n
+    a.t_cap = Kc.t_cap
+    a.idx_bits, a.main_bits, a.aux_bits, a.qmax = Kc.idx_bits, Kc.main_bits, Kc.aux_bits, Kc.qmax
+    keep = None
+    if kv_lens is not None:
+        keep = kv_lens.to(device=dev, dtype=torch.int32).contiguous()
+        a.kv_len = L.ptr(keep)
+    a.causal, a.causal_offset, a.softmax_scale = int(causal), causal_offset, softmax_scale
+    a.n_splits = n_splits
+    ws = None
+    if n_splits > 1:
+        nbytes = int(L.lib().hqmq_attn_workspace_bytes(C.c_int(B), C.c_int(Hq), C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits)))
+        ws = _workspace(nbytes, dev, "attn")
+        a.workspace, a.workspace_bytes = L.ptr(ws), ws.numel()
+    with torch.cuda.device(dev):
+        L.check(L.lib().hqmq_attn_fwd(C.byref(a), L.stream_ptr(dev)), "hqmq_attn_fwd")
+    return O

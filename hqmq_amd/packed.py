@@ -1,0 +1,106 @@
+"""Bit-packed HQMQ cache containers (device memory owned by torch).
+
+PackedTensor holds one tensor (K or V) of one layer: the code planes, the
+per-token scales, the Med3x flag plane and outlier sideband, and the joint
+codebook the codes index.  PackedKV pairs a K and a V PackedTensor.
+Plane layout: include/hqmq_amd.h.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib as L
+
+TILE = 16          # tokens per sideband tile
+T_ALIGN = 64       # plane capacity is rounded up to whole attention super-tiles
+
+
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
+class PackedTensor:
+    """Packed codes of a (B, H, T, d_h) tensor; rows [0, length) are valid."""
+
+    def __init__(self, B: int, H: int, t_cap: int, d_head: int, secondary_size: int, radius_bits: int,
+                 dtype: torch.dtype, device, joint: Optional[torch.Tensor] = None, outliers: bool = False,
+                 sideband_frac: float = 0.125, layout: Optional[tuple] = None):
+        if d_head % 4:
+            raise ValueError(f"d_head={d_head} not divisible by 4")
+        self.B, self.H, self.d_head, self.n = B, H, d_head, d_head // 4
+        self.t_cap = _round_up(max(t_cap, 1), T_ALIGN)
+        self.secondary_size, self.radius_bits = secondary_size, radius_bits
+        self.qmax = (1 << radius_bits) - 1
+        self.dtype, self.device = dtype, torch.device(device)
+        # (idx_bits, main_bits, aux_bits); the default is the tight layout of include/hqmq_amd.h
+        self.idx_bits, self.main_bits, self.aux_bits = layout or L.layout_bits(secondary_size, radius_bits)
+        n = self.n
+        z = dict(dtype=torch.uint8, device=self.device)
+        self.main = torch.zeros(B, H, self.t_cap, (n * self.main_bits + 7) // 8, **z)
+        self.aux = torch.zeros(B, H, self.t_cap, (n * self.aux_bits + 7) // 8, **z) if self.aux_bits else None
+        self.scale = torch.zeros(B, H, self.t_cap, dtype=dtype, device=self.device)
+        self.joint = joint
+        self.length = 0                      # rows written when all sequences advance together
+        self.lengths: Optional[torch.Tensor] = None  # per-sequence rows (int32, device) for ragged batches
+        self.flags = self.sideband = self.sb_tile_off = self.sb_count = self.sb_overflow = None
+        self.sb_cap = 0
+        if outliers:
+            self.flags = torch.zeros(B, H, self.t_cap, (n + 7) // 8, **z)
+            self.sb_cap = max(64, int(self.t_cap * n * sideband_frac))
+            self.sideband = torch.zeros(B, H, self.sb_cap, 4, dtype=dtype, device=self.device)
+            self.sb_tile_off = torch.zeros(B, H, self.t_cap // TILE, dtype=torch.int32, device=self.device)
+            self.sb_count = torch.zeros(B, H, dtype=torch.int32, device=self.device)
+            self.sb_overflow = torch.zeros(1, dtype=torch.int32, device=self.device)
+
+    @property
+    def has_outliers(self) -> bool:
+        return self.flags is not None
+
+    def row_bytes(self) -> float:
+        """Stored bytes per (token, head), excluding sideband entries."""
+        b = self.main.shape[-1] + self.scale.element_size()
+        if self.aux is not None:
+            b += self.aux.shape[-1]
+        if self.flags is not None:
+            b += self.flags.shape[-1]
+        return b
+
+    def nbytes(self, length: Optional[int] = None) -> int:
+        """Algorithmic bytes of the first `length` rows of every (b, h) stream, sideband included."""
+        t = self.length if length is None else length
+        total = self.B * self.H * t * self.row_bytes()
+        if self.sb_count is not None:
+            total += int(self.sb_count.sum().item()) * 4 * self.scale.element_size()
+        return int(total)
+
+    def c_struct(self) -> L.Packed:
+        s = L.Packed()
+        s.main_plane, s.aux_plane, s.flag_plane = L.ptr(self.main), L.ptr(self.aux), L.ptr(self.flags)
+        s.scale_plane = L.ptr(self.scale)
+        s.scale_sb, s.scale_sh, s.scale_st = self.scale.stride(0), self.scale.stride(1), self.scale.stride(2)
+        s.sideband, s.sb_tile_off, s.sb_cap = L.ptr(self.sideband), L.ptr(self.sb_tile_off), self.sb_cap
+        s.joint, s.joint_sh, s.K = L.ptr(self.joint), self.joint.stride(0), self.joint.shape[1]
+        return s
+
+    def check_overflow(self) -> None:
+        """Raises if an append ran out of sideband room (reads one int from the device)."""
+        if self.sb_overflow is not None and int(self.sb_overflow.item()):
+            raise L.HqmqError(f"outlier sideband overflow: more than {self.sb_cap} flagged chunks in one (b, h) stream; "
+                              "allocate the cache with a larger sideband_frac")
+
+
+@dataclass
+class PackedKV:
+    """The compressed K and V of one layer."""
+    K: PackedTensor
+    V: PackedTensor
+
+    @property
+    def length(self) -> int:
+        return self.K.length
+
+    def nbytes(self, length: Optional[int] = None) -> int:
+        return self.K.nbytes(length) + self.V.nbytes(length)

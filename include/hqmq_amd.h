@@ -106,6 +106,11 @@ int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x_stride_h, 
                          int B, int H, int T, int n_chunks, float mult, void *workspace, int64_t workspace_bytes,
                          float *median, void *thr, int32_t *n_out, void *stream);
 
+/* Med3x mask alone, for wrappers around quantizers other than HQMQ: mask[b][h][t][c] = ||chunk|| > thr[h]
+ * (src/quantizers/outlier_generic.py:60 of the reference). One byte per chunk. */
+int hqmq_outlier_mask(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype,
+                      int B, int H, int T, int n_chunks, const void *thr, uint8_t *mask, void *stream);
+
 /* Compact the flagged chunks of rows [row0, row0+T) into the sideband.
  * No counterpart in the reference (its wrapper keeps a dense tensor).
  * Rows must be appended in order; row0 = (pos ? pos[b] : 0) + t_off. */
@@ -144,9 +149,13 @@ typedef struct hqmq_packed {
     int K;                    /* codewords in joint */
 } hqmq_packed;
 
-/* Dense decode of a packed cache (outlier chunks substituted from the sideband). */
+/* Dense decode of a packed cache (outlier chunks substituted from the sideband).
+ * mode 0: cw * ((rq * rs) / qmax), the rounding of _decode_kv_torch
+ *         (src/quantizers/hqmq_attention.py:61-64) that the attention path is checked against;
+ * mode 1: (rq * (rs / qmax)) * cw, the rounding of the quantizer's own output
+ *         (src/quantizers/hqmq.py:210-216). */
 int hqmq_dequant_packed(const hqmq_packed *p, int dtype, int B, int H, int T, int n_chunks, int64_t t_cap,
-                        int idx_bits, int main_bits, int aux_bits, int qmax, void *out, void *stream);
+                        int idx_bits, int main_bits, int aux_bits, int qmax, int mode, void *out, void *stream);
 
 /* Fused attention over the packed cache: decode (T_q = 1) and chunked prefill.
  * Replaces fused_hqmq_attention_triton (src/quantizers/hqmq_attention.py:425-518)

@@ -97,7 +97,8 @@ def outlier_quantize(x, joint, radius_bits: int, mult: float = 3.0) -> dict:
     m = med3x(x, mult)
     merged = torch.empty_like(x)
     mask8 = m["mask"].to(torch.uint8).contiguous()
-    lib().orc_outlier_merge(_p(x.contiguous()), _p(q["out"]), _p(mask8), C.c_int(DT_CODE[x.dtype]),
+    x = x.contiguous()
+    lib().orc_outlier_merge(_p(x), _p(q["out"]), _p(mask8), C.c_int(DT_CODE[x.dtype]),
                             C.c_long(mask8.numel()), _p(merged))
     q.update(m)
     q["inner_out"] = q["out"]
@@ -140,7 +141,8 @@ def pack_rows(idx, rq, idx_bits: int, main_bits: int, aux_bits: int):
     as_ = (n * aux_bits + 7) // 8
     main = torch.empty(rows, ms, dtype=torch.uint8)
     aux = torch.empty(rows, as_, dtype=torch.uint8) if aux_bits else None
-    lib().orc_pack_rows(_p(idx.to(torch.int32).contiguous()), _p(rq.to(torch.int32).contiguous()), C.c_long(rows),
+    idx32, rq32 = idx.to(torch.int32).contiguous(), rq.to(torch.int32).contiguous()  # keep alive across the call
+    lib().orc_pack_rows(_p(idx32), _p(rq32), C.c_long(rows),
                         C.c_int(n), C.c_int(idx_bits), C.c_int(main_bits), C.c_int(aux_bits), _p(main),
                         C.c_long(ms), _p(aux), C.c_long(as_))
     return main.view(*lead, ms), (aux.view(*lead, as_) if aux is not None else None)
@@ -151,7 +153,8 @@ def pack_flags(mask: torch.Tensor) -> torch.Tensor:
     rows = mask.numel() // n
     st = (n + 7) // 8
     flags = torch.empty(rows, st, dtype=torch.uint8)
-    lib().orc_pack_flags(_p(mask.to(torch.uint8).contiguous()), C.c_long(rows), C.c_int(n), _p(flags), C.c_long(st))
+    mask8 = mask.to(torch.uint8).contiguous()  # keep alive across the call
+    lib().orc_pack_flags(_p(mask8), C.c_long(rows), C.c_int(n), _p(flags), C.c_long(st))
     return flags.view(*lead, st)
 
 

@@ -1,0 +1,77 @@
+"""The reference's GPU smoke tests (tests/test_gpu.py there), run against this build's package."""
+import pytest
+import torch
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
+
+
+def test_quantize_on_gpu():
+    import hqmq
+    q = hqmq.HQMQ(n_layers=2, n_heads=2, secondary_size=24, radius_bits=3, device="cuda", init="random")
+    K = torch.randn(1, 2, 16, 128, dtype=torch.bfloat16, device="cuda")
+    Kq = q.quantize_K(K, layer_idx=0)
+    assert Kq.shape == K.shape and Kq.device == K.device and Kq.dtype == K.dtype
+    diff = (K.float() - Kq.float()).abs().mean().item()
+    corr = torch.corrcoef(torch.stack([K.float().flatten(), Kq.float().flatten()]))[0, 1].item()
+    assert diff > 1e-4 and corr > 0.7          # the reference's round-trip sanity bounds (tests/test_smoke.py:178-192)
+
+
+def test_fp32_round_trip_shapes():
+    import hqmq
+    q = hqmq.HQMQ(n_layers=2, n_heads=2, secondary_size=24, radius_bits=3, device="cuda")
+    K = torch.randn(1, 2, 16, 128, dtype=torch.float32, device="cuda")
+    Kq = q.quantize_K(K, layer_idx=0)
+    assert Kq.shape == K.shape and Kq.dtype == K.dtype
+
+
+def test_padded_quantizer_on_gpu():
+    import hqmq
+    p = hqmq.PaddedHQMQ(n_layers=1, n_heads=2, d_head=45, secondary_size=24, radius_bits=3, device="cuda")
+    x = torch.randn(1, 2, 9, 45, device="cuda", dtype=torch.float16)
+    y = p.quantize_K(x, 0)
+    assert y.shape == x.shape
+    padded = torch.nn.functional.pad(x, (0, 3))
+    assert torch.equal(y, p.inner.quantize_K(padded, 0)[..., :45])
+
+
+def test_device_info_reports_real_gpu():
+    import hqmq
+    info = hqmq.device_info()
+    assert info["gpu"] is not None and info["variant_auto_dispatched"] == "cdna4"
+    assert info["arch"].startswith("gfx950")
+
+
+def test_fp8_flag_is_ignored():
+    """use_fp8_codebook=True falls through to the same kernel (the reference's pre-Hopper behaviour)."""
+    import hqmq
+    B, H_q, H_kv, T, dh, S, r_qmax = 1, 4, 1, 32, 32, 24, 7
+    torch.manual_seed(0)
+    Q = torch.randn(B, H_q, T, dh, dtype=torch.float16, device="cuda") * 0.3
+    idx = torch.randint(0, 24 * S, (B, H_kv, T, dh // 4), dtype=torch.int32, device="cuda")
+    rq = torch.randint(1, r_qmax + 1, (B, H_kv, T, dh // 4), dtype=torch.int32, device="cuda")
+    rs = torch.rand((B, H_kv, T), dtype=torch.float16, device="cuda") + 0.5
+    joint = torch.randn((H_kv, 24 * S, 4), dtype=torch.float16, device="cuda")
+    joint = joint / joint.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    a = hqmq.fused_attention(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
+    b = hqmq.fused_attention(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True, use_fp8_codebook=True)
+    assert torch.equal(a, b)
+    from hqmq import kernels
+    c = kernels.fused_attention_hopper(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
+    d = kernels.fused_attention_blackwell(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
+    assert torch.equal(a, c) and torch.equal(a, d)
+
+
+def test_encode_joint_fp8():
+    from hqmq.kernels import encode_joint_fp8
+    joint = torch.randn(2, 24 * 24, 4, dtype=torch.float16, device="cuda")
+    joint = joint / joint.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    j8 = encode_joint_fp8(joint)
+    assert j8.dtype == torch.float8_e4m3fn and j8.shape == joint.shape
+
+
+def test_native_library_is_what_ran():
+    """The kernels come from the in-tree shared library, loaded into this process."""
+    from hqmq_amd import _lib as L
+    so = str(L.library_path())
+    with open("/proc/self/maps") as f:
+        assert any(so in line for line in f)

@@ -1,0 +1,225 @@
+"""GPU parity for the fused attention kernel: golden outputs of the reference's torch path, dense attention
+over the dequantized cache (CPU oracle, double accumulation), and size-independent properties at full size.
+
+Tolerance: |O - ref| <= 2e-3 + 2*eps*|ref| element-wise (1e-3 base for fp32, the reference's own test bound),
+eps = 2^-11 for fp16/fp32 (the kernel multiplies in fp16), 2^-8 for bf16 (the result's own rounding).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as CO
+from oracle import torch_oracle as TO
+from tests.helpers import DT, attn_tolerance, bit_equal, kv_input, unbits
+from tests.test_oracle import ATTN_CASES, load_attn_case
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
+DEV = "cuda"
+
+
+def assert_close(got, ref, dtype, base=2e-3, what=""):
+    ref = ref.float().cpu()
+    err = (got.float().cpu() - ref).abs()
+    tol = attn_tolerance(ref, dtype, base)
+    worst = float((err - tol).max())
+    assert worst <= 0, f"{what}: max abs err {float(err.max()):.3e}, exceeds tolerance by {worst:.3e}"
+
+
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_golden_unpacked_api(case, golden_dir):
+    """hqmq.fused_attention with the reference's argument list against the reference's own torch output."""
+    import hqmq
+    m, t = load_attn_case(np.load(golden_dir / "attention.npz"), case)
+    d = {k: v.to(DEV) for k, v in t.items()}
+    base = 1e-3 if m["dtype"] == torch.float32 else 2e-3
+    for kw in (dict(), dict(n_splits=1), dict(n_splits=3), dict(block_q=64, block_kv=64, num_warps=4, num_stages=2,
+                                                               optimized=False, use_fp8_codebook=True)):
+        O = hqmq.fused_attention(d["Q"], d["K_idx"], d["K_rq"], d["K_rs"], d["K_joint"], d["V_idx"], d["V_rq"],
+                                 d["V_rs"], d["V_joint"], r_qmax=m["qmax"], causal=m["causal"], **kw)
+        assert O.shape == d["Q"].shape and O.dtype == d["Q"].dtype
+        assert_close(O, t["O"], m["dtype"], base, f"{case} {kw}")
+    Oref = hqmq.fused_attention_reference(d["Q"], d["K_idx"], d["K_rq"], d["K_rs"], d["K_joint"], d["V_idx"], d["V_rq"],
+                                          d["V_rs"], d["V_joint"], r_qmax=m["qmax"], causal=m["causal"])
+    assert_close(Oref, t["O"], m["dtype"], base, f"{case} unfused")
+
+
+def test_reference_gpu_test_recipe():
+    """The reference's only numerical kernel test (tests/test_gpu.py:24-49): fp32, causal, max abs diff < 1e-3."""
+    import hqmq
+    B, H_q, H_kv, T, dh, S, r_qmax = 1, 4, 1, 64, 32, 24, 7
+    K_size = 24 * S
+    torch.manual_seed(0)
+    Q = torch.randn(B, H_q, T, dh, dtype=torch.float32, device=DEV) * 0.3
+    idx = torch.randint(0, K_size, (B, H_kv, T, dh // 4), dtype=torch.int32, device=DEV)
+    rq = torch.randint(1, r_qmax + 1, (B, H_kv, T, dh // 4), dtype=torch.int32, device=DEV)
+    rs = torch.rand((B, H_kv, T), dtype=torch.float32, device=DEV) + 0.5
+    joint = torch.randn((H_kv, K_size, 4), dtype=torch.float32, device=DEV)
+    joint = joint / joint.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    O_ref = hqmq.fused_attention_reference(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
+    O_fused = hqmq.fused_attention(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
+    assert (O_ref - O_fused).abs().max().item() < 1e-3
+    cpu = CO.attention_dense(Q.cpu(), CO.dequant(idx.cpu(), rq.cpu(), rs.cpu(), joint.cpu(), r_qmax),
+                             CO.dequant(idx.cpu(), rq.cpu(), rs.cpu(), joint.cpu(), r_qmax), causal=True)
+    assert (cpu - O_fused.cpu()).abs().max().item() < 1e-3
+
+
+def build_cache(q, k, v, outliers):
+    cache = q.new_cache(k.shape[0], k.shape[2], k.shape[3], k.dtype, 0)
+    q.append(cache, k.to(DEV), v.to(DEV), 0)
+    if outliers:
+        cache.K.check_overflow()
+        cache.V.check_overflow()
+    return cache
+
+
+CASES = [
+    # name, B, H_q, H_kv, T_q, T_kv, d_h, S, b_r, dtype, outliers, causal, causal_offset, kv_lens
+    ("config2 shape, fp16 s96_r4", 1, 32, 8, 1, 1000, 128, 96, 4, "fp16", False, False, 0, None),
+    ("config3 shape, fp16 s192_r6 + Med3x", 2, 28, 4, 1, 300, 128, 192, 6, "fp16", True, False, 0, None),
+    ("config4 shape, bf16 s24_r3 + Med3x, ragged", 3, 32, 8, 1, 400, 128, 24, 3, "bf16", True, False, 0, [400, 130, 257]),
+    ("config5 shape, bf16 s96_r4 + Med3x, d_h=64", 2, 64, 8, 1, 777, 64, 96, 4, "bf16", True, False, 0, None),
+    ("square causal prefill", 1, 8, 2, 100, 100, 128, 96, 4, "fp16", False, True, 0, None),
+    ("rectangular causal, top-left aligned", 1, 4, 2, 5, 190, 64, 24, 3, "fp16", False, True, 0, None),
+    ("chunked prefill, bottom-right aligned", 2, 8, 4, 7, 133, 128, 96, 4, "fp16", False, True, 126, None),
+    ("fp32 cache", 2, 4, 2, 3, 90, 32, 96, 4, "fp32", False, False, 0, None),
+    ("d_h=256", 1, 4, 2, 1, 200, 256, 96, 4, "fp16", False, False, 0, None),
+    ("empty and short sequences", 3, 8, 2, 1, 64, 64, 24, 3, "fp16", False, False, 0, [0, 1, 64]),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_attention_matches_dense_oracle(case):
+    import hqmq
+    from hqmq_amd import ops
+    name, B, Hq, Hkv, Tq, Tkv, d_h, S, b_r, dn, outl, causal, off, lens = case
+    dt = DT[dn]
+    seed = sum(map(ord, name))
+    k = kv_input((B, Hkv, Tkv, d_h), dt, seed, lognormal=False, outlier_p=0.02 if outl else 0)
+    v = kv_input((B, Hkv, Tkv, d_h), dt, seed + 1, lognormal=False, outlier_p=0.02 if outl else 0, outlier_gain=(5, 10))
+    Q = torch.randn(B, Hq, Tq, d_h, generator=torch.Generator().manual_seed(seed + 2)).to(dt)
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV)
+    if outl:
+        q = hqmq.with_outlier_extraction(q, C=3.0)
+    cache = build_cache(q, k, v, outl)
+    Kd, Vd = ops.dequant_packed(cache.K, Tkv, 0).cpu(), ops.dequant_packed(cache.V, Tkv, 0).cpu()   # parity-checked elsewhere
+    ref = CO.attention_dense(Q, Kd, Vd, kv_lens=lens, causal=causal, causal_offset=off)
+    base = 1e-3 if dt == torch.float32 else 2e-3
+    outs = []
+    for ns in (1, 2, 0):
+        O = hqmq.fused_attention_packed(Q.to(DEV), cache, causal=causal, causal_offset=off, n_splits=ns, T_kv=Tkv,
+                                        kv_lens=None if lens is None else torch.tensor(lens))
+        assert_close(O, ref, dt, base, f"{name} n_splits={ns}")
+        outs.append(O)
+    if lens is not None and 0 in lens:
+        assert float(outs[0][lens.index(0)].abs().max()) == 0.0      # nothing to attend to -> zeros, not NaN
+
+
+def test_torch_sdpa_agrees_on_the_same_cache():
+    """Dense SDPA on the GPU over the dequantized cache (what BASELINE config 2 names as the check)."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.float16
+    q = hqmq.HQMQ(n_layers=1, n_heads=8, secondary_size=96, radius_bits=4, device=DEV)
+    k, v = kv_input((1, 8, 4096, 128), dt, 1, lognormal=False), kv_input((1, 8, 4096, 128), dt, 2, lognormal=False)
+    cache = build_cache(q, k, v, False)
+    Q = torch.randn(1, 32, 1, 128, generator=torch.Generator().manual_seed(3)).to(dt).to(DEV)
+    Kd, Vd = ops.dequant_packed(cache.K, 4096, 0), ops.dequant_packed(cache.V, 4096, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(Q, Kd.repeat_interleave(4, 1), Vd.repeat_interleave(4, 1))
+    O = hqmq.fused_attention_packed(Q, cache)
+    assert (O.float() - ref.float()).abs().max().item() < 2e-3
+
+
+@pytest.mark.parametrize("T", [4096, 32768])
+def test_config2_full_size_properties(T):
+    """BASELINE config 2 at full size (32 / 8 heads, d_h=128, s96_r4, fp16, one query token):
+    split invariance, zero padding rows ignored, agreement with dense fp32 attention on the GPU, 2e-3 bound."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.float16
+    q = hqmq.HQMQ(n_layers=1, n_heads=8, secondary_size=96, radius_bits=4, device=DEV)
+    g = torch.Generator().manual_seed(T)
+    k, v = torch.randn(1, 8, T, 128, generator=g).to(dt), torch.randn(1, 8, T, 128, generator=g).to(dt)
+    Q = torch.randn(1, 32, 1, 128, generator=g).to(dt).to(DEV)
+    cache = build_cache(q, k, v, False)
+    outs = [hqmq.fused_attention_packed(Q, cache, n_splits=ns) for ns in (0, 1, 7, 64)]
+    for o in outs[1:]:
+        assert (o.float() - outs[0].float()).abs().max().item() < 2e-4       # split-KV merge is exact up to fp32 order
+    Kd, Vd = ops.dequant_packed(cache.K, T, 0).float(), ops.dequant_packed(cache.V, T, 0).float()
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float().view(1, 8, 4, 128), Kd) * 128 ** -0.5
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, dim=-1), Vd).reshape(1, 32, 1, 128)
+    assert (outs[0].float() - ref).abs().max().item() < 2e-3
+    # a sequence-length argument shorter than the cache behaves like a shorter cache
+    half = hqmq.fused_attention_packed(Q, cache, kv_lens=torch.tensor([T // 2]), T_kv=T)
+    s2 = s[..., :T // 2]
+    ref2 = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s2, dim=-1), Vd[:, :, :T // 2]).reshape(1, 32, 1, 128)
+    assert (half.float() - ref2).abs().max().item() < 2e-3
+
+
+def test_decode_loop_with_append_config4_shape():
+    """Config 4 shape in miniature: ragged batch, each step quantize-and-appends one bf16 token per sequence
+    (s24_r3, Med3x) and attends with per-sequence lengths; compared with the oracle after the last step."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.bfloat16
+    B, Hq, Hkv, d_h, steps = 4, 32, 8, 128, 3
+    lens0 = [100, 17, 64, 1]
+    Tmax = max(lens0) + steps
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=24, radius_bits=3, device=DEV))
+    cache = w.new_cache(B, Tmax, d_h, dt, 0, sideband_frac=0.25)
+    k_all = kv_input((B, Hkv, Tmax, d_h), dt, 21, outlier_p=0.02)
+    v_all = kv_input((B, Hkv, Tmax, d_h), dt, 22)
+    pos = torch.tensor(lens0, dtype=torch.int32, device=DEV)
+    # prefill each sequence separately (its own Med3x statistics), then step together
+    ref_k = torch.zeros(B, Hkv, Tmax, d_h, dtype=dt)
+    ref_v = torch.zeros(B, Hkv, Tmax, d_h, dtype=dt)
+    Jk = CO.joint_table(TO.secondary_raw(1, Hkv, 24, 42)[0, :, 0], dt)
+    Jv = CO.joint_table(TO.secondary_raw(1, Hkv, 24, 42)[0, :, 1], dt)
+
+    def oracle_dense(x, J):
+        r = CO.outlier_quantize(x, J, 3, 3.0)
+        n = x.shape[-1] // 4
+        d = CO.dequant(r["idx"], r["rq"], r["r_max"], J, 7).view(*x.shape[:3], n, 4)
+        return torch.where(r["mask"].unsqueeze(-1), x.view(*x.shape[:3], n, 4), d).reshape(x.shape)
+
+    for b, L0 in enumerate(lens0):
+        sub = w.new_cache(1, Tmax, d_h, dt, 0, sideband_frac=0.25)
+        w.append(sub, k_all[b:b + 1, :, :L0].to(DEV), v_all[b:b + 1, :, :L0].to(DEV), 0)
+        for dst, src in ((cache.K, sub.K), (cache.V, sub.V)):
+            for name in ("main", "aux", "scale", "flags", "sideband", "sb_tile_off", "sb_count"):
+                getattr(dst, name)[b] = getattr(src, name)[0]
+        ref_k[b, :, :L0] = oracle_dense(k_all[b:b + 1, :, :L0].contiguous(), Jk)[0]
+        ref_v[b, :, :L0] = oracle_dense(v_all[b:b + 1, :, :L0].contiguous(), Jv)[0]
+    for s in range(steps):
+        idx = (pos.cpu().long()).tolist()
+        k_new = torch.stack([k_all[b, :, idx[b]:idx[b] + 1] for b in range(B)])
+        v_new = torch.stack([v_all[b, :, idx[b]:idx[b] + 1] for b in range(B)])
+        w.append(cache, k_new.to(DEV), v_new.to(DEV), 0, pos=pos)
+        dk, dv = oracle_dense(k_new.contiguous(), Jk), oracle_dense(v_new.contiguous(), Jv)
+        for b in range(B):
+            ref_k[b, :, idx[b]] = dk[b, :, 0]
+            ref_v[b, :, idx[b]] = dv[b, :, 0]
+        pos += 1
+        Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(30 + s)).to(dt)
+        O = hqmq.fused_attention_packed(Q.to(DEV), cache, kv_lens=pos, T_kv=Tmax)
+        ref = CO.attention_dense(Q, ref_k, ref_v, kv_lens=pos.cpu().tolist())
+        assert_close(O, ref, dt, 2e-3, f"step {s}")
+    cache.K.check_overflow()
+    dense = ops.dequant_packed(cache.K, Tmax, 0).cpu()
+    for b, L in enumerate(pos.cpu().tolist()):
+        assert bit_equal(dense[b, :, :L], ref_k[b, :, :L])
+
+
+def test_argument_checks():
+    import hqmq
+    q = hqmq.HQMQ(n_layers=1, n_heads=2, secondary_size=24, radius_bits=3, device=DEV)
+    cache = q.new_cache(1, 64, 64, torch.float16, 0)
+    x = torch.randn(1, 2, 64, 64, device=DEV).half()
+    q.append(cache, x, x, 0)
+    with pytest.raises(AssertionError):
+        hqmq.fused_attention_packed(torch.randn(1, 3, 1, 64, device=DEV).half(), cache)       # H_q % H_kv
+    with pytest.raises(AssertionError):
+        hqmq.fused_attention_packed(torch.randn(1, 4, 1, 32, device=DEV).half(), cache)       # d_h mismatch
+    with pytest.raises(hqmq.HqmqError):
+        hqmq.fused_attention_packed(torch.randn(1, 4, 1, 64, device=DEV), cache)              # dtype mismatch
+    with pytest.raises(hqmq.HqmqError):
+        q.append(cache, x, x, 0)                                                              # capacity exceeded

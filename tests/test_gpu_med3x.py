@@ -1,0 +1,158 @@
+"""GPU parity for Med3x: radix-select median, threshold, mask, flag plane and outlier sideband."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as CO
+from oracle import torch_oracle as TO
+from tests.helpers import DT, bit_equal, kv_input, unbits
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("dn", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 3, 70, 64), (1, 2, 5, 12), (1, 1, 1, 128), (3, 4, 257, 128)])
+def test_median_threshold_count(dn, shape):
+    """Even and odd chunk counts, tiny calls (one decode token), all dtypes (fp32 takes the two-pass select)."""
+    from hqmq_amd import ops
+    dt = DT[dn]
+    x = kv_input(shape, dt, seed=sum(shape), outlier_p=0.04)
+    want = CO.med3x(x, 3.0)
+    med, thr, cnt = ops.med3x_threshold(x.to(DEV), 3.0)
+    assert torch.equal(med.cpu(), want["median"])
+    assert bit_equal(thr, want["threshold"])
+    assert torch.equal(cnt.cpu().long(), want["mask"].sum(dim=(0, 2, 3)))
+    assert torch.equal(ops.outlier_mask(x.to(DEV), thr).cpu(), want["mask"])
+
+
+def test_median_with_duplicates_and_nan():
+    from hqmq_amd import ops
+    x = torch.ones(1, 2, 8, 16).half()           # every norm equal: both middle ranks fall in one bin
+    x[0, 1, :, :] *= torch.arange(1, 9).view(8, 1)
+    want = CO.med3x(x)
+    med, thr, cnt = ops.med3x_threshold(x.to(DEV))
+    assert torch.equal(med.cpu(), want["median"]) and bit_equal(thr, want["threshold"])
+    x[0, 0, 2, 5] = float("nan")                 # a NaN norm makes that head's quantile NaN and its mask empty
+    want = CO.med3x(x)
+    med, thr, cnt = ops.med3x_threshold(x.to(DEV))
+    assert torch.isnan(med[0]).item() and float(med[1]) == float(want["median"][1])
+    assert int(cnt[0]) == 0 and not ops.outlier_mask(x.to(DEV), thr)[:, 0].any()
+
+
+def test_outlier_golden_outputs(golden_dir):
+    """with_outlier_extraction(...).quantize_K/V reproduce the reference's outputs bit for bit; the running
+    outlier rate and bits_per_value match too."""
+    import hqmq
+    g = np.load(golden_dir / "outlier.npz")
+    for cfg in ("s24r3", "s96r4"):
+        S, b_r, seed, L, H = (int(v) for v in g[cfg + "_meta"])
+        inner = hqmq.HQMQ(n_layers=L, n_heads=H, secondary_size=S, radius_bits=b_r, device=DEV, seed=seed)
+        for dn, dt in DT.items():
+            w = hqmq.with_outlier_extraction(inner, C=3.0)
+            for kv, tag in ((0, "K"), (1, "V")):
+                key = f"{cfg}_{dn}_{tag}"
+                x = unbits(g[key + "_x"], dt).to(DEV)
+                y = w.quantize_K(x, 0) if kv == 0 else w.quantize_V(x, 0)
+                assert bit_equal(y, unbits(g[key + "_out"], dt)), key
+            rate, n_obs, bpv = g[f"{cfg}_{dn}_rate"]
+            assert abs(w.bits_per_value() - bpv) < 1e-6
+            assert w._n_observations == int(n_obs) and abs(w._observed_outlier_rate - rate) < 1e-7
+
+
+def test_generic_wrapper_matches_hqmq_wrapper():
+    import hqmq
+    q = hqmq.HQMQ(n_layers=1, n_heads=2, secondary_size=24, radius_bits=3, device=DEV)
+    x = kv_input((2, 2, 40, 64), torch.float16, seed=4, outlier_p=0.05).to(DEV)
+    a = hqmq.with_outlier_extraction(q, C=3.0).quantize_K(x, 0)
+    b = hqmq.with_outlier_extraction(q, C=3.0, generic=True).quantize_K(x, 0)
+    assert bit_equal(a, b)
+
+
+@pytest.mark.parametrize("S,b_r,dn,d_h", [(24, 3, "bf16", 128), (96, 4, "bf16", 64), (192, 6, "fp16", 128), (24, 3, "fp32", 32)])
+def test_flags_and_sideband_match_oracle(S, b_r, dn, d_h):
+    """Bulk quantize with Med3x into the packed cache: flag plane, sideband order, tile offsets, counts, and
+    the dense decode with outliers substituted."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = DT[dn]
+    B, H, T = 2, 2, 150
+    n = d_h // 4
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=S, radius_bits=b_r, device=DEV, seed=5))
+    k = kv_input((B, H, T, d_h), dt, seed=S, outlier_p=0.03)
+    v = kv_input((B, H, T, d_h), dt, seed=S + 1, outlier_p=0.01, outlier_gain=(5, 10))
+    cache = w.new_cache(B, T, d_h, dt, 0)
+    w.append(cache, k.to(DEV), v.to(DEV), 0)
+    cache.K.check_overflow()
+    for pt, x, kv in ((cache.K, k, 0), (cache.V, v, 1)):
+        Jc = CO.joint_table(TO.secondary_raw(1, H, S, 5)[0, :, kv], dt)
+        want = CO.outlier_quantize(x, Jc, b_r, 3.0)
+        assert int(want["mask"].sum()) > 0
+        assert torch.equal(pt.flags[:, :, :T].cpu(), CO.pack_flags(want["mask"]))
+        for b in range(B):
+            for h in range(H):
+                sb, toff, cnt = CO.pack_sideband(x[b, h], want["mask"][b, h])
+                assert int(pt.sb_count[b, h]) == cnt
+                assert bit_equal(pt.sideband[b, h, :cnt], sb)
+                assert torch.equal(pt.sb_tile_off[b, h, :toff.numel()].cpu(), toff)
+        assert bit_equal(ops.dequant_packed(pt, T, mode=1), want["out"])
+        dense = CO.dequant(want["idx"], want["rq"], want["r_max"], Jc, pt.qmax).view(B, H, T, n, 4)
+        dense = torch.where(want["mask"].unsqueeze(-1), x.view(B, H, T, n, 4), dense).reshape(B, H, T, d_h)
+        assert bit_equal(ops.dequant_packed(pt, T, mode=0), dense)
+    assert cache.nbytes() == sum(pt.B * pt.H * T * pt.row_bytes() + int(pt.sb_count.sum()) * 4 * pt.scale.element_size()
+                                 for pt in (cache.K, cache.V))
+
+
+def test_decode_appends_keep_sideband_consistent():
+    """Token-by-token appends (each call has its own per-head median, as the reference's cache hook does)
+    leave the same planes as the oracle run call by call, across tile boundaries."""
+    import hqmq
+    dt = torch.bfloat16
+    B, H, d_h, steps = 4, 2, 128, 37
+    n = d_h // 4
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=24, radius_bits=3, device=DEV))
+    cache = w.new_cache(B, steps, d_h, dt, 0, sideband_frac=0.5)
+    ks = kv_input((B, H, steps, d_h), dt, seed=7, outlier_p=0.05)
+    vs = kv_input((B, H, steps, d_h), dt, seed=8)
+    for t in range(steps):
+        w.append(cache, ks[:, :, t:t + 1].to(DEV), vs[:, :, t:t + 1].to(DEV), 0)
+    cache.K.check_overflow()
+    Jc = CO.joint_table(TO.secondary_raw(1, H, 24, 42)[0, :, 0], dt)
+    masks = torch.cat([CO.med3x(ks[:, :, t:t + 1].contiguous())["mask"] for t in range(steps)], dim=2)
+    assert torch.equal(cache.K.flags[:, :, :steps].cpu(), CO.pack_flags(masks))
+    for b in range(B):
+        for h in range(H):
+            sb, toff, cnt = CO.pack_sideband(ks[b, h], masks[b, h])
+            assert int(cache.K.sb_count[b, h]) == cnt and bit_equal(cache.K.sideband[b, h, :cnt], sb)
+            assert torch.equal(cache.K.sb_tile_off[b, h, :toff.numel()].cpu(), toff)
+    assert w._n_observations == 0 and len(w._pending) == 2 * steps     # no device sync per call
+    w.bits_per_value()
+    assert w._n_observations == 2 * steps
+
+
+def test_sideband_overflow_is_reported():
+    import hqmq
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=1, secondary_size=24, radius_bits=3, device=DEV))
+    cache = w.new_cache(1, 512, 128, torch.float16, 0, sideband_frac=0.001)   # room for 64 chunks only
+    x = kv_input((1, 1, 512, 128), torch.float16, seed=3, outlier_p=0.2).to(DEV)
+    w.append(cache, x, x, 0)
+    with pytest.raises(hqmq.HqmqError):
+        cache.K.check_overflow()
+
+
+def test_full_size_median_properties():
+    """Config-3 scale per head (8.4 M chunk norms): the selected median splits the norms in half and the
+    count above the threshold equals a direct count (size-independent properties; no CPU sort of 8 M values
+    per head in the test)."""
+    from hqmq_amd import ops
+    x = kv_input((8, 2, 32768, 128), torch.float16, seed=11, lognormal=False, outlier_p=0.02).to(DEV)
+    med, thr, cnt = ops.med3x_threshold(x, 3.0)
+    mask = ops.outlier_mask(x, thr)                      # direct count vs the histogram-derived count
+    assert torch.equal(mask.sum(dim=(0, 2, 3)).to(torch.int32), cnt)
+    norms = x.view(8, 2, 32768, 32, 4).float().norm(dim=-1)    # torch on the GPU, approximate: for the split check only
+    for h in range(2):
+        nh = norms[:, h].reshape(-1)
+        N = nh.numel()
+        slack = N // 1000                                        # torch's norm may round a few values the other way
+        assert int((nh < med[h]).sum()) <= N // 2 + slack and int((nh > med[h]).sum()) <= N // 2 + slack
+    assert 0.01 < float(cnt.sum()) / norms.numel() < 0.04
