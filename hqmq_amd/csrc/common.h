@@ -27,7 +27,12 @@ struct F16 {
     static constexpr int code = HQMQ_F16;
     static __device__ __forceinline__ float load(const storage *p) { return __half2float(__ushort_as_half(*p)); }
     static __device__ __forceinline__ void store(storage *p, float f) { *p = __half_as_ushort(__float2half_rn(f)); }
-    static __device__ __forceinline__ float rnd(float f) { return __half2float(__float2half_rn(f)); }
+    // The empty asm keeps the fp32 value opaque: without it the compiler folds a preceding fused
+    // multiply-add into v_fma_mixlo_f16, which rounds once to fp16 instead of fp32-then-fp16.
+    static __device__ __forceinline__ float rnd(float f) {
+        asm volatile("" : "+v"(f));
+        return __half2float(__float2half_rn(f));
+    }
     static __device__ __forceinline__ float eps() { return 4.8828125e-4f; }  // 2^-11
 };
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {

