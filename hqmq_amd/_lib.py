@@ -56,7 +56,7 @@ class AttnArgs(C.Structure):
         ("T_kv", C.c_int), ("n_chunks", C.c_int), ("t_cap", i64),
         ("idx_bits", C.c_int), ("main_bits", C.c_int), ("aux_bits", C.c_int), ("qmax", C.c_int),
         ("kv_len", vp), ("causal", C.c_int), ("causal_offset", i64), ("softmax_scale", C.c_float),
-        ("n_splits", C.c_int), ("workspace", vp), ("workspace_bytes", i64),
+        ("n_splits", C.c_int), ("workspace", vp), ("workspace_bytes", i64), ("skip_combine", C.c_int), ("force_generic", C.c_int),
     ]
 
 
@@ -64,7 +64,7 @@ EXPORTS = [
     "hqmq_version", "hqmq_status_string", "hqmq_layout_bits", "hqmq_build_joint", "hqmq_quantize",
     "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",
     "hqmq_pack_codes", "hqmq_dequant_packed", "hqmq_attn_workspace_bytes", "hqmq_attn_pick_splits",
-    "hqmq_attn_fwd",
+    "hqmq_attn_fwd", "hqmq_attn_combine",
 ]
 
 

@@ -48,7 +48,7 @@ def _pack_unpacked(idx, rq, rs, joint, r_qmax: int) -> PackedTensor:
     pt = PackedTensor(B, H, T, 4 * n, S_eff, rb, joint.dtype, idx.device, joint=joint, layout=(ib, mb, ab))
     pt.qmax = int(r_qmax)
     ops.pack_codes(idx, rq, pt)
-    pt.scale = rs.to(joint.dtype)      # (B, H, T), any strides: the kernels take them explicitly
+    pt.scale[:, :, :T] = rs            # into the padded plane: rows up to the capacity stay readable
     pt.length = T
     return pt
 

@@ -18,163 +18,40 @@
 //   * KV is walked in super-tiles of 64 tokens; each lane reads its codes with one aligned
 //     vector load per 16-token tile, a wavefront covering whole 128-byte lines of the plane;
 //   * split-KV partials (m, l, acc) go to a workspace and are merged by a second kernel.
-#include "common.h"
+#include "attention_common.h"
 
 namespace hqmq {
 
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-constexpr int kAttnWaves = 4;
-constexpr int kSuper = 64;  // tokens per super-tile
-
-struct PackedDev {
-    const uint8_t *main_plane, *aux_plane, *flag_plane;
-    const void *scale_plane;
-    int64_t ssb, ssh, sst;
-    const void *sideband;
-    const int32_t *sb_tile_off;
-    int64_t sb_cap;
-    const void *joint;
-    int64_t jsh;
-    int K;
+// Raw codes, aux bits and per-token scales of one 64-token super-tile, as one lane needs them:
+// K side (token = lane % 16 of each tile, code group = lane / 16) and V side (token = 4*(lane/16) + lane%4,
+// code group = (lane % 16) / 4); scales of the 4 tokens 4*(lane/16) + 0..3 of each tile (S^T / P^T rows).
+template <int NW>
+struct SuperTile {
+    uint32_t kw[4][NW], vw[4][NW];
+    uint64_t kaux[4], vaux[4];
+    float ks[4][4], vs[4][4];
 };
 
-struct AttnParams {
-    const void *Q;
-    void *O;
-    int64_t qsb, qsh, qst, osb, osh, ost;
-    PackedDev Kc, Vc;
-    int dtype;
-    int B, Hq, Hkv, G, Tq, Tkv, n;
-    int64_t t_cap;
-    int idx_bits, aux_bits, qmax;
-    const int32_t *kv_len;
-    int causal;
-    int64_t causal_offset;
-    float c_log2;   // softmax_scale * log2(e) / qmax
-    float c_plain;  // softmax_scale * log2(e)
-    float inv_qmax;
-    int n_splits, n_cg;
-    float *ws;
-};
-
-__device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {
-    if (dtype == HQMQ_F16) return __half2float(__ushort_as_half(((const uint16_t *)p)[i]));
-    if (dtype == HQMQ_BF16) return __uint_as_float((uint32_t)((const uint16_t *)p)[i] << 16);
-    return ((const float *)p)[i];
-}
-__device__ __forceinline__ void store_any(void *p, int dtype, int64_t i, float f) {
-    if (dtype == HQMQ_F16) ((uint16_t *)p)[i] = __half_as_ushort(__float2half_rn(f));
-    else if (dtype == HQMQ_BF16) ((uint16_t *)p)[i] = f32_to_bf16_bits(f);
-    else ((float *)p)[i] = f;
-}
-__device__ __forceinline__ half4 load_chunk_h(const void *p, int dtype, int64_t chunk) {
-    half4 r;
-    if (dtype == HQMQ_F16) {
-        const uint2 w = *reinterpret_cast<const uint2 *>((const uint16_t *)p + chunk * 4);
-        r = __builtin_bit_cast(half4, w);
-    } else {
-        for (int j = 0; j < 4; j++) r[j] = (_Float16)load_any(p, dtype, chunk * 4 + j);
-    }
-    return r;
-}
-
-// The lane's NB = CPL*MB/8 bytes of main-plane codes, as 32-bit words.
-template <int NB>
-__device__ __forceinline__ void load_bytes(const uint8_t *p, uint32_t (&w)[(NB + 3) / 4]) {
-    constexpr int NW = (NB + 3) / 4;
-    if constexpr (NB % 16 == 0) {
-        for (int i = 0; i < NB / 16; i++) {
-            const uint4 v = reinterpret_cast<const uint4 *>(p)[i];
-            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+__device__ __forceinline__ void load_scales4(const void *plane, int dtype, int64_t base, int64_t st, bool vec, int t, int Tkv,
+                                             float (&out)[4]) {
+    if (vec) {  // 4 consecutive tokens, t % 4 == 0, rows up to the plane capacity are readable
+        if (dtype == HQMQ_F32) {
+            const float4 v = *reinterpret_cast<const float4 *>((const float *)plane + base + t);
+            out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2 *>((const uint16_t *)plane + base + t);
+            if (dtype == HQMQ_F16) {
+                const half4 h = __builtin_bit_cast(half4, v);
+                out[0] = (float)h[0]; out[1] = (float)h[1]; out[2] = (float)h[2]; out[3] = (float)h[3];
+            } else {
+                out[0] = __uint_as_float(v.x << 16); out[1] = __uint_as_float(v.x & 0xffff0000u);
+                out[2] = __uint_as_float(v.y << 16); out[3] = __uint_as_float(v.y & 0xffff0000u);
+            }
         }
-    } else if constexpr (NB % 8 == 0) {
-        for (int i = 0; i < NB / 8; i++) {
-            const uint2 v = reinterpret_cast<const uint2 *>(p)[i];
-            w[2 * i] = v.x; w[2 * i + 1] = v.y;
-        }
-    } else if constexpr (NB % 4 == 0) {
-        for (int i = 0; i < NW; i++) w[i] = reinterpret_cast<const uint32_t *>(p)[i];
-    } else if constexpr (NB % 2 == 0) {
-        for (int i = 0; i < NW; i++) w[i] = 0;
-        for (int i = 0; i < NB / 2; i++) w[i >> 1] |= (uint32_t) reinterpret_cast<const uint16_t *>(p)[i] << (16 * (i & 1));
     } else {
-        for (int i = 0; i < NW; i++) w[i] = 0;
-        for (int i = 0; i < NB; i++) w[i >> 2] |= (uint32_t)p[i] << (8 * (i & 3));
+#pragma unroll
+        for (int e = 0; e < 4; e++) out[e] = (t + e < Tkv) ? load_any(plane, dtype, base + (int64_t)(t + e) * st) : 0.f;
     }
-}
-
-template <int MB, int NW>
-__device__ __forceinline__ uint32_t code_at(const uint32_t (&w)[NW], int j) {
-    const int pos = j * MB, wd = pos >> 5, sh = pos & 31;
-    uint32_t v = w[wd] >> sh;
-    if (sh + MB > 32 && wd + 1 < NW) v |= w[wd + 1] << (32 - sh);
-    return v & ((1u << MB) - 1u);
-}
-
-// aux bits of the lane's CPL codes: bits [first_code*ab, (first_code+CPL)*ab) of the aux row
-template <int CPL>
-__device__ __forceinline__ uint64_t load_aux(const uint8_t *row, int row_bytes, int first_code, int ab) {
-    const int start = first_code * ab, nbits = CPL * ab;
-    const int b0 = start >> 3, sh = start & 7;
-    uint64_t v = 0;
-    for (int i = 0; i * 8 < nbits + sh && b0 + i < row_bytes && i < 8; i++) v |= (uint64_t)row[b0 + i] << (8 * i);
-    v >>= sh;
-    if (nbits + sh > 64 && b0 + 8 < row_bytes) v |= (uint64_t)row[b0 + 8] << (64 - sh);
-    return v;
-}
-
-__device__ __forceinline__ uint32_t dpp_quad_xor2(uint32_t v) {  // lane i <- lane i^2 within each quad
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
-}
-__device__ __forceinline__ uint32_t dpp_quad_xor1(uint32_t v) {  // lane i <- lane i^1
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
-}
-
-// Quad lane i holds (e(i,0), e(i,1)) in r0 and (e(i,2), e(i,3)) in r1; afterwards lane i holds
-// (e(0,i), e(1,i)) in r0 and (e(2,i), e(3,i)) in r1.
-__device__ __forceinline__ void quad_transpose(uint32_t &r0, uint32_t &r1, int lane) {
-    const bool upper = lane & 2;
-    const uint32_t send = upper ? r0 : r1;
-    const uint32_t recv = dpp_quad_xor2(send);
-    const uint32_t X = upper ? recv : r0, Y = upper ? r1 : recv;
-    const uint32_t PX = dpp_quad_xor1(X), PY = dpp_quad_xor1(Y);
-    const uint32_t sel = (lane & 1) ? 0x03020706u : 0x05040100u;
-    r0 = __builtin_amdgcn_perm(PX, X, sel);
-    r1 = __builtin_amdgcn_perm(PY, Y, sel);
-}
-
-
-// Flag bookkeeping for one 16-token tile. Every lane passes the token it decodes (`tok`, 0..15)
-// and the first chunk of its code group; returns the lane's CPL flag bits and the sideband slot
-// of its first flagged chunk: tile offset + flagged chunks of earlier tokens + earlier chunks.
-template <int CPL>
-__device__ __forceinline__ void tile_flags(const PackedDev &c, size_t plane_row0, int64_t tile_row, int64_t t_cap, int frb,
-                                           size_t tile_off_index, int col, int tok, int first, uint32_t &fl, int &slot0) {
-    int64_t row = tile_row + col;
-    if (row >= t_cap) row = t_cap - 1;
-    uint32_t fw = 0;
-    const uint8_t *fr = c.flag_plane + (plane_row0 + row) * frb;
-    for (int i = 0; i < frb && i < 4; i++) fw |= (uint32_t)fr[i] << (8 * i);
-    const int own = __popc(fw);
-    int pre = own;
-    for (int o = 1; o < 16; o <<= 1) {
-        const int v = __shfl_up(pre, o, 16);
-        if (col >= o) pre += v;
-    }
-    pre -= own;                          // flagged chunks in tokens < col of this tile
-    const uint32_t fw_t = (uint32_t)__shfl((int)fw, tok, 16);
-    const int pre_t = __shfl(pre, tok, 16);
-    fl = (fw_t >> first) & ((CPL >= 32) ? 0xffffffffu : ((1u << CPL) - 1u));
-    slot0 = c.sb_tile_off[tile_off_index] + pre_t + __popc(fw_t & ((first >= 32) ? 0xffffffffu : ((1u << first) - 1u)));
-}
-
-// A flagged chunk: the verbatim values from the sideband (exact in fp16 for fp16 caches).
-__device__ __forceinline__ half4 outlier_chunk(const PackedDev &c, int dtype, size_t bh, int slot) {
-    int64_t s = slot;
-    if (s >= c.sb_cap) s = c.sb_cap - 1;
-    return load_chunk_h(c.sideband, dtype, (int64_t)bh * c.sb_cap + s);
 }
 
 template <int CPL, int MB, bool FLAGS>
@@ -184,27 +61,64 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + p.Kc.K;
 
-    const int bh = blockIdx.y, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
+    const int bh = blockIdx.z, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
+    const int cg = blockIdx.y, sp = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int dtype = p.dtype;
-
-    // ---- per-head codeword tables -> LDS as fp16 ----
-    for (int k = threadIdx.x; k < p.Kc.K; k += blockDim.x)
-        ktab[k] = __builtin_bit_cast(uint2, load_chunk_h(p.Kc.joint, dtype, hkv * (p.Kc.jsh / 4) + k));
-    for (int k = threadIdx.x; k < p.Vc.K; k += blockDim.x)
-        vtab[k] = __builtin_bit_cast(uint2, load_chunk_h(p.Vc.joint, dtype, hkv * (p.Vc.jsh / 4) + k));
-    __syncthreads();
-
-    const int item = blockIdx.x * kAttnWaves + wave;
-    if (item >= p.n_cg * p.n_splits) return;
-    const int cg = item / p.n_splits, sp = item - cg * p.n_splits;
-
     const int n = p.n, G = p.G;
     const int col = lane & 15, grp = lane >> 4;
     const int cidx = cg * 16 + col;
     const bool col_ok = cidx < p.Tq * G;
     const int tq = col_ok ? cidx / G : 0, g = col_ok ? cidx - tq * G : 0;
     const int hq = hkv * G + g;
+
+    // ---- KV range of this block and of this wave ----
+    int kv_end = p.kv_len ? p.kv_len[b] : p.Tkv;
+    kv_end = min(max(kv_end, 0), p.Tkv);
+    int64_t lim64 = kv_end;                       // per-column visible limit (exclusive)
+    if (p.causal) lim64 = min(lim64, (int64_t)tq + p.causal_offset + 1);
+    if (!col_ok || lim64 < 0) lim64 = 0;
+    const int col_lim = (int)lim64;
+    int blk_lim = col_lim;                        // block-wide limit: max over the 16 columns
+    for (int o = 1; o < 16; o <<= 1) blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
+    int per_split = (blk_lim + p.n_splits - 1) / p.n_splits;
+    per_split = (per_split + kSuper - 1) / kSuper * kSuper;
+    const int b_begin = min(sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
+    int per_wave = (b_end - b_begin + kAttnWaves - 1) / kAttnWaves;
+    per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
+    const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
+
+    const size_t plane_row0 = (size_t)bh * p.t_cap;
+    const int mrb = n * MB / 8;
+    const int arb = (n * p.aux_bits + 7) >> 3;
+    const int frb = (n + 7) >> 3;
+    const int64_t tiles_cap = (p.t_cap + kTile - 1) / kTile;
+    const uint32_t idx_mask = (1u << p.idx_bits) - 1u;
+    const int idx_bits = p.idx_bits, ab = p.aux_bits;
+    const int v_tok = 4 * grp + (col & 3), v_grp = col >> 2;   // V-side lane role
+    const int64_t ks_base = b * p.Kc.ssb + hkv * p.Kc.ssh, vs_base = b * p.Vc.ssb + hkv * p.Vc.ssh;
+
+    auto load_super = [&](int t0, SuperTile<NW> &s) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int64_t krow = min((int64_t)t0 + 16 * u + col, p.t_cap - 1);
+            const int64_t vrow = min((int64_t)t0 + 16 * u + v_tok, p.t_cap - 1);
+            load_bytes<NB>(p.Kc.main_plane + (plane_row0 + krow) * mrb + grp * NB, s.kw[u]);
+            load_bytes<NB>(p.Vc.main_plane + (plane_row0 + vrow) * mrb + v_grp * NB, s.vw[u]);
+            s.kaux[u] = s.vaux[u] = 0;
+            if (ab) {
+                s.kaux[u] = load_aux<CPL>(p.Kc.aux_plane + (plane_row0 + krow) * arb, arb, grp * CPL, ab);
+                s.vaux[u] = load_aux<CPL>(p.Vc.aux_plane + (plane_row0 + vrow) * arb, arb, v_grp * CPL, ab);
+            }
+            const int ts = t0 + 16 * u + 4 * grp;
+            load_scales4(p.Kc.scale_plane, dtype, ks_base, p.Kc.sst, p.scale_vec, ts, p.Tkv, s.ks[u]);
+            load_scales4(p.Vc.scale_plane, dtype, vs_base, p.Vc.sst, p.scale_vec, ts, p.Tkv, s.vs[u]);
+        }
+    };
+
+    // the first super-tile's loads fly while the codeword tables are copied to LDS
+    SuperTile<NW> cur;
+    if (t_begin < t_end) load_super(t_begin, cur);
 
     // ---- Q^T fragment: lane (col, grp) holds dims [grp*CPL*4, +CPL*4) of its column ----
     half4 qf[CPL];
@@ -217,54 +131,25 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
         }
     }
 
-    // ---- KV range of this item ----
-    int kv_end = p.kv_len ? p.kv_len[b] : p.Tkv;
-    if (kv_end > p.Tkv) kv_end = p.Tkv;
-    if (kv_end < 0) kv_end = 0;
-    // per-column visible limit (exclusive)
-    int64_t lim64 = kv_end;
-    if (p.causal) {
-        const int64_t cl = (int64_t)tq + p.causal_offset + 1;
-        if (cl < lim64) lim64 = cl;
-    }
-    if (!col_ok || lim64 < 0) lim64 = 0;
-    const int col_lim = (int)lim64;
-    // wave-wide limit: max over the 16 columns (columns are ordered by query token)
-    int wave_lim = col_lim;
-    for (int o = 1; o < 16; o <<= 1) wave_lim = max(wave_lim, __shfl_xor(wave_lim, o));
-    int per_split = (wave_lim + p.n_splits - 1) / p.n_splits;
-    per_split = (per_split + kSuper - 1) / kSuper * kSuper;
-    const int t_begin = sp * per_split;
-    const int t_end = min(wave_lim, t_begin + per_split);
-
-    const size_t plane_row0 = (size_t)bh * p.t_cap;
-    const int mrb = n * MB / 8;
-    const int arb = (n * p.aux_bits + 7) >> 3;
-    const int frb = (n + 7) >> 3;
-    const int64_t tiles_cap = (p.t_cap + kTile - 1) / kTile;
-    const uint32_t idx_mask = (1u << p.idx_bits) - 1u;
-    const int idx_bits = p.idx_bits, ab = p.aux_bits;
+    // ---- per-head codeword tables -> LDS as fp16 ----
+    fill_table(ktab, p.Kc.joint, dtype, hkv * (p.Kc.jsh / 4), p.Kc.K);
+    fill_table(vtab, p.Vc.joint, dtype, hkv * (p.Vc.jsh / 4), p.Vc.K);
+    __syncthreads();
 
     float m_run = -INFINITY, l_run = 0.f;
     float4v acc[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // K-side lane role: token = col (row of the A operand), code group = grp
-    // V-side lane role: token = 4*grp + (col & 3), code group = col >> 2
-    const int v_tok = 4 * grp + (col & 3), v_grp = col >> 2;
-
     for (int t0 = t_begin; t0 < t_end; t0 += kSuper) {
+        SuperTile<NW> nxt;
+        const bool more = t0 + kSuper < t_end;
+        if (more) load_super(t0 + kSuper, nxt);
+
         float4v sT[4], sTo[4];
         // ---------------- S^T = K . Q^T for 4 tiles ----------------
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            int64_t row = (int64_t)t0 + 16 * u + col;
-            if (row >= p.t_cap) row = p.t_cap - 1;
-            uint32_t w[NW];
-            load_bytes<NB>(p.Kc.main_plane + (plane_row0 + row) * mrb + grp * NB, w);
-            uint64_t aux = 0;
-            if (ab) aux = load_aux<CPL>(p.Kc.aux_plane + (plane_row0 + row) * arb, arb, grp * CPL, ab);
             uint32_t fl = 0;
             int sb_base = 0;
             if (FLAGS)
@@ -273,8 +158,8 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
             float4v s = float4v{0.f, 0.f, 0.f, 0.f}, so = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < CPL; j++) {
-                uint32_t code = code_at<MB, NW>(w, j);
-                if (ab) code |= (uint32_t)((aux >> (j * ab)) & ((1u << ab) - 1u)) << MB;
+                uint32_t code = code_at<MB, NW>(cur.kw[u], j);
+                if (ab) code |= (uint32_t)((cur.kaux[u] >> (j * ab)) & ((1u << ab) - 1u)) << MB;
                 const uint32_t k = code & idx_mask;
                 const _Float16 rq = (_Float16)(float)(code >> idx_bits);
                 half4 a = __builtin_bit_cast(half4, ktab[k]);
@@ -304,9 +189,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + 16 * u + 4 * grp + e;
-                float rs = 0.f;
-                if (t < p.Tkv) rs = load_any(p.Kc.scale_plane, dtype, b * p.Kc.ssb + hkv * p.Kc.ssh + (int64_t)t * p.Kc.sst);
-                float v = sT[u][e] * (rs * p.c_log2);
+                float v = sT[u][e] * (cur.ks[u][e] * p.c_log2);
                 if (FLAGS) v = fmaf(sTo[u][e], p.c_plain, v);
                 v = (t < col_lim && t < t_end) ? v : -INFINITY;
                 pv[u][e] = v;
@@ -329,23 +212,13 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
             for (int e = 0; e < 4; e++) {
                 const float pe = exp2f(pv[u][e] - m_use);
                 l_run += pe;
-                const int t = t0 + 16 * u + 4 * grp + e;
-                float rs = 0.f;
-                if (t < p.Tkv) rs = load_any(p.Vc.scale_plane, dtype, b * p.Vc.ssb + hkv * p.Vc.ssh + (int64_t)t * p.Vc.sst);
-                pT[u][e] = (_Float16)(pe * (rs * p.inv_qmax));
+                pT[u][e] = (_Float16)(pe * (cur.vs[u][e] * p.inv_qmax));
                 if (FLAGS) pTo[u][e] = (_Float16)pe;
-                pv[u][e] = pe;
             }
         }
         // ---------------- O^T += V^T . P^T ----------------
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            int64_t row = (int64_t)t0 + 16 * u + v_tok;
-            if (row >= p.t_cap) row = p.t_cap - 1;
-            uint32_t w[NW];
-            load_bytes<NB>(p.Vc.main_plane + (plane_row0 + row) * mrb + v_grp * NB, w);
-            uint64_t aux = 0;
-            if (ab) aux = load_aux<CPL>(p.Vc.aux_plane + (plane_row0 + row) * arb, arb, v_grp * CPL, ab);
             uint32_t fl = 0;
             int sb_base = 0;
             if (FLAGS)
@@ -353,8 +226,8 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
                                 (size_t)bh * tiles_cap + min((int64_t)((t0 + 16 * u) >> 4), tiles_cap - 1), col, v_tok, v_grp * CPL, fl, sb_base);
 #pragma unroll
             for (int j = 0; j < CPL; j++) {
-                uint32_t code = code_at<MB, NW>(w, j);
-                if (ab) code |= (uint32_t)((aux >> (j * ab)) & ((1u << ab) - 1u)) << MB;
+                uint32_t code = code_at<MB, NW>(cur.vw[u], j);
+                if (ab) code |= (uint32_t)((cur.vaux[u] >> (j * ab)) & ((1u << ab) - 1u)) << MB;
                 const uint32_t k = code & idx_mask;
                 const _Float16 rq = (_Float16)(float)(code >> idx_bits);
                 half4 a = __builtin_bit_cast(half4, vtab[k]);
@@ -377,52 +250,91 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
                 acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, r), pT[u], acc[j], 0, 0, 0);
             }
         }
+        if (more) cur = nxt;
     }
 
-    // ---- epilogue: lane (col, grp) holds, for block j, dims 4*(CPL*grp + j) + 0..3 of column col ----
+    // ---- merge the block's waves through LDS (the tables are no longer needed) ----
+    // lane (col, grp) holds, for block j, dims 4*(CPL*grp + j) + 0..3 of column col
     float l_tot = l_run;
     l_tot += __shfl_xor(l_tot, 16);
     l_tot += __shfl_xor(l_tot, 32);
-    if (!col_ok) return;
-    if (p.n_splits == 1) {
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        const int64_t base = b * p.osb + hq * p.osh + (int64_t)tq * p.ost + grp * CPL * 4;
-#pragma unroll
-        for (int j = 0; j < CPL; j++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) store_any(p.O, dtype, base + 4 * j + e, acc[j][e] * inv);
-    } else {
-        const int d_h = 4 * n;
-        float *wp = p.ws + ((((size_t)b * p.Hq + hq) * p.Tq + tq) * p.n_splits + sp) * (size_t)(d_h + 2);
+    const int d_h = 4 * n;
+    float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][d_h + 2]
+    __syncthreads();
+    {
+        float *wp = red + ((size_t)wave * 16 + col) * (d_h + 2);
         if (grp == 0) { wp[0] = m_run; wp[1] = l_tot; }
 #pragma unroll
         for (int j = 0; j < CPL; j++)
 #pragma unroll
             for (int e = 0; e < 4; e++) wp[2 + grp * CPL * 4 + 4 * j + e] = acc[j][e];
     }
-}
-
-// One thread per output element; merges the split partials of its row.
-__global__ void attn_combine_kernel(const float *ws, void *O, int dtype, int B, int Hq, int Tq, int d_h, int n_splits,
-                                    int64_t osb, int64_t osh, int64_t ost) {
-    const int64_t total = (int64_t)B * Hq * Tq * d_h;
-    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (int64_t)gridDim.x * blockDim.x) {
-        const int e = (int)(g % d_h);
-        const int64_t row = g / d_h;
-        const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
-        const float *wp = ws + (size_t)row * n_splits * (d_h + 2);
+    __syncthreads();
+    for (int o = threadIdx.x; o < 16 * d_h; o += blockDim.x) {
+        const int c = o / d_h, e = o - c * d_h;
+        const int ci = cg * 16 + c;
+        if (ci >= p.Tq * G) continue;
         float m = -INFINITY;
-        for (int s = 0; s < n_splits; s++) m = fmaxf(m, wp[(size_t)s * (d_h + 2)]);
-        float l = 0.f, o = 0.f;
+        for (int w = 0; w < kAttnWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + c) * (d_h + 2)]);
+        float l = 0.f, a = 0.f;
         if (m > -INFINITY) {
-            for (int s = 0; s < n_splits; s++) {
-                const float *q = wp + (size_t)s * (d_h + 2);
-                const float w = exp2f(q[0] - m);
-                l += q[1] * w;
-                o += q[2 + e] * w;
+            for (int w = 0; w < kAttnWaves; w++) {
+                const float *q = red + ((size_t)w * 16 + c) * (d_h + 2);
+                const float f = exp2f(q[0] - m);
+                l = fmaf(q[1], f, l);
+                a = fmaf(q[2 + e], f, a);
             }
         }
-        store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, l > 0.f ? o / l : 0.f);
+        const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
+        if (p.n_splits == 1) {
+            store_any(p.O, dtype, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a / l : 0.f);
+        } else {
+            float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
+            if (e == 0) { wp[0] = m; wp[1] = l; }
+            wp[2 + e] = a;
+        }
+    }
+}
+
+// One 256-thread block per output row: splits are spread over the threads, then reduced through LDS.
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
+                                                           int n_splits, int64_t osb, int64_t osh, int64_t ost) {
+    __shared__ float m_sh[512];
+    __shared__ float part[256 + 8];
+    __shared__ float l_part[8];
+    const int64_t row = blockIdx.x;
+    const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
+    const float *wp = ws + (size_t)row * n_splits * (d_h + 2);
+    float m = -INFINITY;
+    for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
+        const float v = wp[(size_t)s * (d_h + 2)];
+        if (s < 512) m_sh[s] = v;
+        m = fmaxf(m, v);
+    }
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if ((threadIdx.x & 63) == 0) part[256 + (threadIdx.x >> 6)] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(part[256], part[257]), fmaxf(part[258], part[259]));
+    __syncthreads();
+    // threads = (element e, split phase ph); d_h <= 256
+    const int lanes_e = d_h, phases = 256 / lanes_e > 8 ? 8 : 256 / lanes_e;
+    const int e = threadIdx.x % lanes_e, ph = threadIdx.x / lanes_e;
+    float o = 0.f, l = 0.f;
+    if (m > -INFINITY && ph < phases) {
+        for (int s = ph; s < n_splits; s += phases) {
+            const float *q = wp + (size_t)s * (d_h + 2);
+            const float w = exp2f((s < 512 ? m_sh[s] : q[0]) - m);
+            o = fmaf(q[2 + e], w, o);
+            if (e == 0) l = fmaf(q[1], w, l);
+        }
+    }
+    part[threadIdx.x] = o;
+    if (e == 0 && ph < 8) l_part[ph] = l;
+    __syncthreads();
+    if (ph == 0) {
+        float lt = 0.f;
+        for (int k = 0; k < phases && k < 8; k++) { lt += l_part[k]; if (k) o += part[k * lanes_e + e]; }
+        store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, lt > 0.f ? o / lt : 0.f);
     }
 }
 
@@ -463,16 +375,30 @@ extern "C" int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, i
     return (int64_t)B * H_q * T_q * n_splits * (d_h + 2) * 4;
 }
 
+// Blocks per (sequence, KV head, column group): enough blocks to put two on every CU, each block's four
+// wavefronts keeping at least one 64-token super-tile.
 extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv) {
     if (B < 1 || H_q < 1 || H_kv < 1 || T_q < 1 || T_kv < 1) return 1;
     const int G = H_q / H_kv;
     const int64_t base = (int64_t)B * H_kv * ((T_q * G + 15) / 16);
-    int64_t s = (2048 + base - 1) / base;
-    const int64_t cap = (T_kv + 2 * kSuper - 1) / (2 * kSuper);
+    int64_t s = (512 + base - 1) / base;
+    const int64_t cap = (T_kv + kAttnWaves * kSuper - 1) / (kAttnWaves * kSuper);
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     if (s > 512) s = 512;
     return (int)s;
+}
+
+extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,
+                                 int64_t o_sb, int64_t o_sh, int64_t o_st, void *stream) {
+    if (!workspace || !O) return HQMQ_ERR_NULL;
+    if (B < 1 || H_q < 1 || T_q < 1 || d_h < 4 || d_h > 256 || (d_h & (d_h - 1)) || n_splits < 1) return HQMQ_ERR_SHAPE;
+    if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
+    const int64_t rows = (int64_t)B * H_q * T_q;
+    if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (const float *)workspace, O,
+                       dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
+    return hip_status(hipGetLastError());
 }
 
 extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
@@ -501,12 +427,16 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if (flags && (((uintptr_t)a->K.sideband % (4 * elt)) || ((uintptr_t)a->V.sideband % (4 * elt)))) return HQMQ_ERR_ALIGN;
 
     int n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv);
+    if (n_splits > 65535) return HQMQ_ERR_SHAPE;
     if (n_splits > 1) {
         if (!a->workspace) return HQMQ_ERR_NULL;
         if (a->workspace_bytes < hqmq_attn_workspace_bytes(a->B, a->H_q, a->T_q, 4 * n, n_splits)) return HQMQ_ERR_WORKSPACE;
         if ((uintptr_t)a->workspace & 3) return HQMQ_ERR_ALIGN;
     }
-    const size_t shmem = ((size_t)a->K.K + a->V.K) * 8;
+    // LDS: the two fp16 codeword tables, reused afterwards for the cross-wave merge
+    size_t shmem = ((size_t)a->K.K + a->V.K) * 8;
+    const size_t merge = (size_t)kAttnWaves * 16 * (4 * n + 2) * sizeof(float);
+    if (shmem < merge) shmem = merge;
     if (shmem > 152 * 1024) return HQMQ_ERR_SHAPE;
 
     AttnParams p;
@@ -524,11 +454,23 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     p.n_splits = n_splits;
     p.n_cg = (a->T_q * p.G + 15) / 16;
     p.ws = (float *)a->workspace;
-    const int64_t items = (int64_t)p.n_cg * n_splits;
-    dim3 grid((unsigned)((items + kAttnWaves - 1) / kAttnWaves), (unsigned)(a->B * a->H_kv));
+    // 4 consecutive scales with one vector load: unit stride, aligned rows, and capacity rows readable
+    const int salign = a->dtype == HQMQ_F32 ? 16 : 8;
+    p.scale_vec = 1;
+    for (const hqmq_packed *k : pk)
+        if (k->scale_st != 1 || (k->scale_sb % 4) || (k->scale_sh % 4) || ((uintptr_t)k->scale_plane % salign) ||
+            k->scale_sh < a->t_cap || (a->t_cap % kSuper))
+            p.scale_vec = 0;
+    if (p.n_cg > 65535) return HQMQ_ERR_SHAPE;
+    dim3 grid((unsigned)n_splits, (unsigned)p.n_cg, (unsigned)(a->B * a->H_kv));
     hipStream_t st = (hipStream_t)stream;
-    int rc;
-    switch (n / 4) {
+    int rc = HQMQ_OK;
+    bool handled = false;
+    if (p.scale_vec && !a->force_generic) {
+        rc = launch_attn_fast(p, a->main_bits, flags, grid, shmem, st, &handled);
+        if (rc) return rc;
+    }
+    if (!handled) switch (n / 4) {
         case 1: rc = launch_attn_mb<1>(p, a->main_bits, flags, grid, shmem, st); break;
         case 2: rc = launch_attn_mb<2>(p, a->main_bits, flags, grid, shmem, st); break;
         case 4: rc = launch_attn_mb<4>(p, a->main_bits, flags, grid, shmem, st); break;
@@ -537,13 +479,8 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
         default: return HQMQ_ERR_SHAPE;
     }
     if (rc) return rc;
-    if (n_splits > 1) {
-        const int64_t total = (int64_t)a->B * a->H_q * a->T_q * 4 * n;
-        int64_t g = (total + 255) / 256;
-        if (g > 1 << 20) g = 1 << 20;
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)g), dim3(256), 0, st, (const float *)a->workspace, a->O,
-                           a->dtype, a->B, a->H_q, a->T_q, 4 * n, n_splits, a->o_sb, a->o_sh, a->o_st);
-        rc = hip_status(hipGetLastError());
-    }
+    if (n_splits > 1 && !a->skip_combine)
+        rc = hqmq_attn_combine(a->workspace, a->O, a->dtype, a->B, a->H_q, a->T_q, 4 * n, n_splits, a->o_sb, a->o_sh, a->o_st,
+                               stream);
     return rc;
 }

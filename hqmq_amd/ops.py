@@ -223,7 +223,8 @@ def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int) -> int:
 
 def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None, causal: bool = False,
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+             out: Optional[torch.Tensor] = None, skip_combine: bool = False,
+             force_generic: bool = False) -> torch.Tensor:
     """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each)."""
     L.require_gpu(Q, "Q")
     if Q.stride(-1) != 1:
@@ -256,6 +257,8 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
         a.kv_len = L.ptr(keep)
     a.causal, a.causal_offset, a.softmax_scale = int(causal), causal_offset, softmax_scale
     a.n_splits = n_splits
+    a.skip_combine = int(skip_combine)
+    a.force_generic = int(force_generic)
     ws = None
     if n_splits > 1:
         nbytes = int(L.lib().hqmq_attn_workspace_bytes(C.c_int(B), C.c_int(Hq), C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits)))

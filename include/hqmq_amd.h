@@ -177,10 +177,15 @@ typedef struct hqmq_attn_args {
     float softmax_scale;
     int n_splits;             /* 0 = choose */
     void *workspace; int64_t workspace_bytes;
+    int skip_combine;         /* 1: leave the split partials in the workspace (merge later with hqmq_attn_combine) */
+    int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
 int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv);
 int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream);
+/* Merge of the split-KV partials (m, l, acc) left in the workspace; hqmq_attn_fwd runs it unless skip_combine. */
+int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,
+                      int64_t o_sb, int64_t o_sh, int64_t o_st, void *stream);
 
 #ifdef __cplusplus
 }
