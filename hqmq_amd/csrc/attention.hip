@@ -296,46 +296,48 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     }
 }
 
-// One 256-thread block per output row: splits are spread over the threads, then reduced through LDS.
+// One block per output row (d_h <= 256 threads used): weights of the splits go to LDS first, then every thread
+// walks the partials of its element with independent loads.
 __global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
                                                            int n_splits, int64_t osb, int64_t osh, int64_t ost) {
-    __shared__ float m_sh[512];
-    __shared__ float part[256 + 8];
-    __shared__ float l_part[8];
+    extern __shared__ float wsh[];          // [n_splits] weights
+    __shared__ float red_m[4], red_l[4];
     const int64_t row = blockIdx.x;
     const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
     const float *wp = ws + (size_t)row * n_splits * (d_h + 2);
     float m = -INFINITY;
-    for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
+    for (int s = threadIdx.x; s < n_splits; s += 256) {
         const float v = wp[(size_t)s * (d_h + 2)];
-        if (s < 512) m_sh[s] = v;
+        wsh[s] = v;
         m = fmaxf(m, v);
     }
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if ((threadIdx.x & 63) == 0) part[256 + (threadIdx.x >> 6)] = m;
+    if ((threadIdx.x & 63) == 0) red_m[threadIdx.x >> 6] = m;
     __syncthreads();
-    m = fmaxf(fmaxf(part[256], part[257]), fmaxf(part[258], part[259]));
-    __syncthreads();
-    // threads = (element e, split phase ph); d_h <= 256
-    const int lanes_e = d_h, phases = 256 / lanes_e > 8 ? 8 : 256 / lanes_e;
-    const int e = threadIdx.x % lanes_e, ph = threadIdx.x / lanes_e;
-    float o = 0.f, l = 0.f;
-    if (m > -INFINITY && ph < phases) {
-        for (int s = ph; s < n_splits; s += phases) {
-            const float *q = wp + (size_t)s * (d_h + 2);
-            const float w = exp2f((s < 512 ? m_sh[s] : q[0]) - m);
-            o = fmaf(q[2 + e], w, o);
-            if (e == 0) l = fmaf(q[1], w, l);
-        }
+    m = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+    float l = 0.f;
+    for (int s = threadIdx.x; s < n_splits; s += 256) {
+        const float f = m > -INFINITY ? exp2f(wsh[s] - m) : 0.f;
+        wsh[s] = f;
+        l = fmaf(wp[(size_t)s * (d_h + 2) + 1], f, l);
     }
-    part[threadIdx.x] = o;
-    if (e == 0 && ph < 8) l_part[ph] = l;
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    if ((threadIdx.x & 63) == 0) red_l[threadIdx.x >> 6] = l;
     __syncthreads();
-    if (ph == 0) {
-        float lt = 0.f;
-        for (int k = 0; k < phases && k < 8; k++) { lt += l_part[k]; if (k) o += part[k * lanes_e + e]; }
-        store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, lt > 0.f ? o / lt : 0.f);
+    l = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
+    const int e = threadIdx.x;
+    if (e >= d_h) return;
+    const float *we = wp + 2 + e;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int s = 0;
+    for (; s + 4 <= n_splits; s += 4) {
+        a0 = fmaf(we[(size_t)(s + 0) * (d_h + 2)], wsh[s + 0], a0);
+        a1 = fmaf(we[(size_t)(s + 1) * (d_h + 2)], wsh[s + 1], a1);
+        a2 = fmaf(we[(size_t)(s + 2) * (d_h + 2)], wsh[s + 2], a2);
+        a3 = fmaf(we[(size_t)(s + 3) * (d_h + 2)], wsh[s + 3], a3);
     }
+    for (; s < n_splits; s++) a0 = fmaf(we[(size_t)s * (d_h + 2)], wsh[s], a0);
+    store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, l > 0.f ? ((a0 + a1) + (a2 + a3)) / l : 0.f);
 }
 
 static PackedDev to_dev(const hqmq_packed &k) {
@@ -375,14 +377,14 @@ extern "C" int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, i
     return (int64_t)B * H_q * T_q * n_splits * (d_h + 2) * 4;
 }
 
-// Blocks per (sequence, KV head, column group): enough blocks to put two on every CU, each block's four
-// wavefronts keeping at least one 64-token super-tile.
+// Blocks per (sequence, KV head, column group): one block per CU, each of a block's eight wavefronts
+// keeping at least one 64-token super-tile.
 extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv) {
     if (B < 1 || H_q < 1 || H_kv < 1 || T_q < 1 || T_kv < 1) return 1;
     const int G = H_q / H_kv;
     const int64_t base = (int64_t)B * H_kv * ((T_q * G + 15) / 16);
-    int64_t s = (512 + base - 1) / base;
-    const int64_t cap = (T_kv + kAttnWaves * kSuper - 1) / (kAttnWaves * kSuper);
+    int64_t s = (256 + base - 1) / base;
+    const int64_t cap = (T_kv + 8 * kSuper - 1) / (8 * kSuper);
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     if (s > 512) s = 512;
@@ -392,11 +394,12 @@ extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv
 extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,
                                  int64_t o_sb, int64_t o_sh, int64_t o_st, void *stream) {
     if (!workspace || !O) return HQMQ_ERR_NULL;
-    if (B < 1 || H_q < 1 || T_q < 1 || d_h < 4 || d_h > 256 || (d_h & (d_h - 1)) || n_splits < 1) return HQMQ_ERR_SHAPE;
+    if (B < 1 || H_q < 1 || T_q < 1 || d_h < 4 || d_h > 256 || (d_h & (d_h - 1)) || n_splits < 1 || n_splits > 8192) return HQMQ_ERR_SHAPE;
     if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (const float *)workspace, O,
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(256), (size_t)n_splits * sizeof(float), (hipStream_t)stream,
+                       (const float *)workspace, O,
                        dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
 }
@@ -427,7 +430,7 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if (flags && (((uintptr_t)a->K.sideband % (4 * elt)) || ((uintptr_t)a->V.sideband % (4 * elt)))) return HQMQ_ERR_ALIGN;
 
     int n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv);
-    if (n_splits > 65535) return HQMQ_ERR_SHAPE;
+    if (n_splits > 8192) return HQMQ_ERR_SHAPE;   // the merge keeps one weight per split in LDS
     if (n_splits > 1) {
         if (!a->workspace) return HQMQ_ERR_NULL;
         if (a->workspace_bytes < hqmq_attn_workspace_bytes(a->B, a->H_q, a->T_q, 4 * n, n_splits)) return HQMQ_ERR_WORKSPACE;
@@ -466,8 +469,8 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     int rc = HQMQ_OK;
     bool handled = false;
-    if (p.scale_vec && !a->force_generic) {
-        rc = launch_attn_fast(p, a->main_bits, flags, grid, shmem, st, &handled);
+    if (p.scale_vec && !a->force_generic && a->softmax_scale > 0.f) {
+        rc = launch_attn_fast(p, a->main_bits, flags, grid, ((size_t)a->K.K + a->V.K) * 8, st, &handled);
         if (rc) return rc;
     }
     if (!handled) switch (n / 4) {

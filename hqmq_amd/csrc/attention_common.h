@@ -39,7 +39,7 @@ struct AttnParams {
     float inv_qmax;
     int n_splits, n_cg;
     int scale_vec;  // scales of 4 consecutive tokens may be read with one aligned vector load
-    float *ws;
+    float *ws;      // split partials [row][split][d_h + 2]
 };
 
 __device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {
@@ -184,6 +184,6 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
 // Implemented in attention_fast.hip: kernels specialised at compile time for the common layouts
 // (d_h 64/128, fp16/bf16 caches, 16+0 / 12+1 / 16+3 bit codes). Returns HQMQ_OK and sets *handled when
 // it launched one of them; otherwise the caller falls back to the generic kernel.
-int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t shmem, hipStream_t st, bool *handled);
+int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled);
 
 }  // namespace hqmq

@@ -22,23 +22,28 @@ __device__ __forceinline__ half4 chunk_to_half(uint2 w) {
     return r;
 }
 
-template <int DT>
-__device__ __forceinline__ void fill_table16(uint2 *dst, const uint2 *src, int K) {
-    constexpr int U = 6;
-    for (int k0 = threadIdx.x; k0 < K; k0 += 256 * U) {
-        uint2 tmp[U];
+// Both per-head tables -> LDS as fp16; every load of the block is in flight before the first store.
+template <int DT, int NT>
+__device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, int Kk, uint2 *vdst, const uint2 *vsrc, int Kv) {
+    constexpr int U = 5;
+    for (int k0 = threadIdx.x; k0 < max(Kk, Kv); k0 += NT * U) {
+        uint2 tk[U], tv[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int k = k0 + u * 256;
-            tmp[u] = k < K ? src[k] : uint2{0, 0};
+            const int k = k0 + u * NT;
+            tk[u] = k < Kk ? ksrc[k] : uint2{0, 0};
+            tv[u] = k < Kv ? vsrc[k] : uint2{0, 0};
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int k = k0 + u * 256;
-            if (k < K) dst[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tmp[u]));
+            const int k = k0 + u * NT;
+            if (k < Kk) kdst[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tk[u]));
+            if (k < Kv) vdst[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tv[u]));
         }
     }
 }
+
+constexpr int kFastWaves = 8;
 
 // codes, aux bits and raw 16-bit scales of one 64-token super-tile for one lane
 template <int NW, int AB>
@@ -56,14 +61,67 @@ __device__ __forceinline__ uint32_t load_small(const uint8_t *p) {
     return v;
 }
 
-template <int CPL, int MB, int AB, int DT, bool FLAGS>
-__global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParams p) {
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// two 16-bit scales (raw bits of dtype DT) as fp32 / as a packed fp16 pair
+template <int DT>
+__device__ __forceinline__ float scale_f32(uint32_t pair, int hi) {
+    if (DT == HQMQ_F16) return (float)__builtin_bit_cast(half2v, pair)[hi];
+    return __uint_as_float(hi ? (pair & 0xffff0000u) : (pair << 16));
+}
+template <int DT>
+__device__ __forceinline__ half2v scale_h2(uint32_t pair) {
+    if (DT == HQMQ_F16) return __builtin_bit_cast(half2v, pair);
+    half2v r;
+    r[0] = (_Float16)__uint_as_float(pair << 16);
+    r[1] = (_Float16)__uint_as_float(pair & 0xffff0000u);
+    return r;
+}
+
+// The V table sits at a fixed LDS offset so that its gathers use the instruction's immediate offset.
+constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
+
+// Decodes the CPL chunks of one lane: gather from the LDS table (byte offset `tab`), times the radius code.
+// 16+0 layout: the two radius codes of a dword become an fp16 pair with one shift, one and-or
+// (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract; the two table addresses take a
+// shift and a mask each.  IB = idx_bits when known at compile time (12 for s96), else 0.
+template <int CPL, int MB, int AB, int IB, int NW>
+__device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t aux, const char *tab, int idx_bits_rt,
+                                              half4 (&a)[CPL]) {
+    const int idx_bits = IB ? IB : idx_bits_rt;
+    const uint32_t idx_mask = (1u << idx_bits) - 1u;
+    if constexpr (MB == 16 && AB == 0) {
+        const uint32_t rq2 = (0xffffu >> idx_bits) * 0x00010001u;
+        const uint2 *t2 = reinterpret_cast<const uint2 *>(tab);
+#pragma unroll
+        for (int i = 0; i < CPL / 2; i++) {
+            const uint32_t lo = w[i] & idx_mask, hi = (w[i] >> 16) & idx_mask;      // and / bit-field extract
+            const uint32_t t = ((w[i] >> idx_bits) & rq2) | 0x64006400u;
+            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
+            a[2 * i] = __builtin_bit_cast(half4, t2[lo]) * r[0];
+            a[2 * i + 1] = __builtin_bit_cast(half4, t2[hi]) * r[1];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < CPL; j++) {
+            uint32_t code = code_at<MB, NW>(w, j);
+            if (AB) code |= ((aux >> (j * AB)) & ((1u << AB) - 1u)) << MB;
+            const _Float16 rq = (_Float16)(uint16_t)(code >> idx_bits);
+            a[j] = __builtin_bit_cast(half4, reinterpret_cast<const uint2 *>(tab)[code & idx_mask]) * rq;
+        }
+    }
+}
+
+template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS>
+__global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParams p) {
     constexpr int NB = CPL * MB / 8;
     constexpr int NW = (NB + 3) / 4;
     constexpr int ABYTES = CPL * AB / 8;     // aux bytes per lane (CPL * AB is a multiple of 8 here)
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
+    constexpr int NT = kFastWaves * 64;
     extern __shared__ uint2 lds_tab[];
-    uint2 *ktab = lds_tab, *vtab = lds_tab + p.Kc.K;
+    uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
+    const char *ktab_b = reinterpret_cast<const char *>(lds_tab), *vtab_b = ktab_b + kVTabOffset;
 
     const int bh = blockIdx.z, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
     const int cg = blockIdx.y, sp = blockIdx.x;
@@ -82,19 +140,21 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
     if (p.causal) lim64 = min(lim64, (int64_t)tq + p.causal_offset + 1);
     if (!col_ok || lim64 < 0) lim64 = 0;
     const int col_lim = (int)lim64;
-    int blk_lim = col_lim;
-    for (int o = 1; o < 16; o <<= 1) blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
+    int blk_lim = col_lim, lim_min = col_ok ? col_lim : 0x7fffffff;
+    for (int o = 1; o < 16; o <<= 1) {
+        blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
+        lim_min = min(lim_min, __shfl_xor(lim_min, o));
+    }
     int per_split = (blk_lim + p.n_splits - 1) / p.n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
-    int per_wave = (b_end - b_begin + kAttnWaves - 1) / kAttnWaves;
+    int per_wave = (b_end - b_begin + kFastWaves - 1) / kFastWaves;
     per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
 
     const size_t plane_row0 = (size_t)bh * p.t_cap;
     constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8, frb = (n + 7) / 8;
     const int64_t tiles_cap = (p.t_cap + kTile - 1) / kTile;
-    const uint32_t idx_mask = (1u << p.idx_bits) - 1u;
     const int idx_bits = p.idx_bits;
     const int v_tok = 4 * grp + (col & 3), v_grp = col >> 2;
     const uint16_t *ks_plane = (const uint16_t *)p.Kc.scale_plane + b * p.Kc.ssb + hkv * p.Kc.ssh;
@@ -133,29 +193,23 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
             qf[j] = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 4 * j)) : half4{0, 0, 0, 0};
     }
 
-    fill_table16<DT>(ktab, (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), p.Kc.K);
-    fill_table16<DT>(vtab, (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4), p.Vc.K);
+    fill_tables16<DT, NT>(ktab, (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), p.Kc.K,
+                          vtab, (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4), p.Vc.K);
     __syncthreads();
 
+    // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
+    const float c = p.c_log2, qmaxf = (float)p.qmax;
     float m_run = -INFINITY, l_run = 0.f;
     float4v acc[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
-
-    auto decode = [&](const uint32_t (&w)[NW], uint32_t aux, int j, const uint2 *tab) -> half4 {
-        uint32_t code = code_at<MB, NW>(w, j);
-        if (AB) code |= ((aux >> (j * AB)) & ((1u << AB) - 1u)) << MB;
-        const _Float16 rq = (_Float16)(uint16_t)(code >> idx_bits);
-        half4 a = __builtin_bit_cast(half4, tab[code & idx_mask]);
-        return a * rq;
-    };
 
     for (int t0 = t_begin; t0 < t_end; t0 += kSuper) {
         FastTile<NW, AB> nxt;
         const bool more = t0 + kSuper < t_end;
         if (more) load_super(t0 + kSuper, nxt);
 
-        float4v sT[4], sTo[4];
+        float4v sT[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             uint32_t fl = 0;
@@ -164,8 +218,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
                 tile_flags<CPL>(p.Kc, plane_row0, (int64_t)t0 + 16 * u, p.t_cap, frb,
                                 (size_t)bh * tiles_cap + min((int64_t)((t0 + 16 * u) >> 4), tiles_cap - 1), col, col, grp * CPL, fl, sb_base);
             half4 a[CPL];
-#pragma unroll
-            for (int j = 0; j < CPL; j++) a[j] = decode(cur.kw[u], AB ? cur.kaux[u] : 0u, j, ktab);
+            decode_chunks<CPL, MB, AB, IB, NW>(cur.kw[u], AB ? cur.kaux[u] : 0u, ktab_b, idx_bits, a);
             float4v s = float4v{0.f, 0.f, 0.f, 0.f}, so = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < CPL; j++) {
@@ -182,48 +235,55 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
                 }
                 s = __builtin_amdgcn_mfma_f32_16x16x16f16(a[j], qf[j], s, 0, 0, 0);
             }
-            sT[u] = s;
-            if (FLAGS) sTo[u] = so;
-        }
-        // ---- scale, mask, online softmax ----
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const uint32_t raw[2] = {cur.ks[u].x, cur.ks[u].y};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int t = t0 + 16 * u + 4 * grp + e;
-                const float rs = cvt16<DT>((raw[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-                float v = sT[u][e] * (rs * p.c_log2);
-                if (FLAGS) v = fmaf(sTo[u][e], p.c_plain, v);
-                v = (t < col_lim && t < t_end) ? v : -INFINITY;
-                sT[u][e] = v;
-                tmax = fmaxf(tmax, v);
+                const float rs = scale_f32<DT>(e < 2 ? cur.ks[u].x : cur.ks[u].y, e & 1);
+                s[e] = s[e] * rs;
+                if (FLAGS) s[e] = fmaf(so[e], qmaxf, s[e]);
             }
+            sT[u] = s;
         }
+        // ---- mask (boundary super-tiles only), online softmax ----
+        if (!(t0 + kSuper <= lim_min && t0 + kSuper <= t_end)) {
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int t = t0 + 16 * u + 4 * grp + e;
+                    if (!(t < col_lim && t < t_end)) sT[u][e] = -INFINITY;
+                }
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(sT[0][0], sT[0][1]), fmaxf(sT[0][2], sT[0][3])),
+                           fmaxf(fmaxf(sT[1][0], sT[1][1]), fmaxf(sT[1][2], sT[1][3])));
+        tmax = fmaxf(tmax, fmaxf(fmaxf(fmaxf(sT[2][0], sT[2][1]), fmaxf(sT[2][2], sT[2][3])),
+                                 fmaxf(fmaxf(sT[3][0], sT[3][1]), fmaxf(sT[3][2], sT[3][3]))));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
         const float m_new = fmaxf(m_run, tmax);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2f(m_run - m_use);
-        m_run = m_new;
-        l_run *= alpha;
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {     // rescale only when some column's maximum moved
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+            l_run *= alpha;
 #pragma unroll
-        for (int j = 0; j < CPL; j++) acc[j] = acc[j] * alpha;
+            for (int j = 0; j < CPL; j++) acc[j] = acc[j] * alpha;
+            m_run = m_new;
+        }
+        const float mc = -m_use * c;
         half4 pT[4], pTo[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const uint32_t raw[2] = {cur.vs[u].x, cur.vs[u].y};
+            float pe[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const float pe = exp2f(sT[u][e] - m_use);
-                l_run += pe;
-                const float rs = cvt16<DT>((raw[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-                pT[u][e] = (_Float16)(pe * (rs * p.inv_qmax));
-                if (FLAGS) pTo[u][e] = (_Float16)pe;
+                pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[u][e], c, mc));
+                l_run += pe[e];
             }
+            const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(cur.vs[u].x);
+            const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(cur.vs[u].y);
+            pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
+            if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
         }
-        // ---- O^T += V^T . P^T ----
+        // ---- O^T += V^T . P^T (the 1/qmax of the radius is applied once, in the epilogue) ----
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             uint32_t fl = 0;
@@ -232,8 +292,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
                 tile_flags<CPL>(p.Vc, plane_row0, (int64_t)t0 + 16 * u, p.t_cap, frb,
                                 (size_t)bh * tiles_cap + min((int64_t)((t0 + 16 * u) >> 4), tiles_cap - 1), col, v_tok, v_grp * CPL, fl, sb_base);
             half4 a[CPL];
-#pragma unroll
-            for (int j = 0; j < CPL; j++) a[j] = decode(cur.vw[u], AB ? cur.vaux[u] : 0u, j, vtab);
+            decode_chunks<CPL, MB, AB, IB, NW>(cur.vw[u], AB ? cur.vaux[u] : 0u, vtab_b, idx_bits, a);
 #pragma unroll
             for (int j = 0; j < CPL; j++) {
                 if (FLAGS) {
@@ -257,7 +316,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
         if (more) cur = nxt;
     }
 
-    // ---- merge the block's waves through LDS, then write the output or this block's partial ----
+    // ---- merge the block's waves through LDS ----
     float l_tot = l_run;
     l_tot += __shfl_xor(l_tot, 16);
     l_tot += __shfl_xor(l_tot, 32);
@@ -272,66 +331,75 @@ __global__ __launch_bounds__(kAttnWaves * 64, 2) void attn_fast_kernel(AttnParam
             for (int e = 0; e < 4; e++) wp[2 + grp * CPL * 4 + 4 * j + e] = acc[j][e];
     }
     __syncthreads();
-    for (int o = threadIdx.x; o < 16 * d_h; o += kAttnWaves * 64) {
-        const int c = o / d_h, e = o - c * d_h;
-        const int ci = cg * 16 + c;
-        if (ci >= p.Tq * G) continue;
+    const int ncols = min(16, p.Tq * G - cg * 16);
+    const float inv_qmax = p.inv_qmax;
+    for (int o = threadIdx.x; o < ncols * d_h; o += NT) {
+        const int cc = o / d_h, e = o - cc * d_h;
+        const int ci = cg * 16 + cc;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kAttnWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + c) * (d_h + 2)]);
+        for (int w = 0; w < kFastWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * (d_h + 2)]);
         float l = 0.f, a = 0.f;
         if (m > -INFINITY) {
 #pragma unroll
-            for (int w = 0; w < kAttnWaves; w++) {
-                const float *q = red + ((size_t)w * 16 + c) * (d_h + 2);
-                const float f = exp2f(q[0] - m);
+            for (int w = 0; w < kFastWaves; w++) {
+                const float *q = red + ((size_t)w * 16 + cc) * (d_h + 2);
+                const float f = __builtin_amdgcn_exp2f((q[0] - m) * c);
                 l = fmaf(q[1], f, l);
                 a = fmaf(q[2 + e], f, a);
             }
         }
         const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
         if (p.n_splits == 1) {
-            store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a / l : 0.f);
+            store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
         } else {
+            // partials carry the maximum in softmax units (base-2 exponent) and acc already divided by qmax
             float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
-            if (e == 0) { wp[0] = m; wp[1] = l; }
-            wp[2 + e] = a;
+            if (e == 0) { wp[0] = m * c; wp[1] = l; }
+            wp[2 + e] = a * inv_qmax;
         }
     }
 }
 
-template <int CPL, int MB, int AB, int DT>
-static int launch_one(const AttnParams &p, bool flags, dim3 grid, size_t shmem, hipStream_t st) {
-    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, DT, true> : attn_fast_kernel<CPL, MB, AB, DT, false>;
+template <int CPL, int MB, int AB, int IB, int DT>
+static int launch_one(const AttnParams &p, bool flags, dim3 grid, size_t table_bytes, hipStream_t st) {
+    // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
+    (void)table_bytes;
+    size_t shmem = (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 2) * sizeof(float);
+    if (shmem < merge) shmem = merge;
+    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true> : attn_fast_kernel<CPL, MB, AB, IB, DT, false>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(kAttnWaves * 64), shmem, st, p);
+    hipLaunchKernelGGL(kern, grid, dim3(kFastWaves * 64), shmem, st, p);
     return hip_status(hipGetLastError());
 }
 
 template <int CPL, int DT>
-static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, size_t shmem, hipStream_t st, bool *handled) {
+static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled) {
+    if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
     *handled = true;
-    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, DT>(p, flags, grid, shmem, st);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, DT>(p, flags, grid, shmem, st);
-    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, DT>(p, flags, grid, shmem, st);
+    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, table_bytes, st);
+    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, table_bytes, st);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, table_bytes, st);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, table_bytes, st);
     *handled = false;
     return HQMQ_OK;
 }
 
-int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t shmem, hipStream_t st, bool *handled) {
+int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled) {
     *handled = false;
     if (p.dtype != HQMQ_F16 && p.dtype != HQMQ_BF16) return HQMQ_OK;
     if (p.n != 16 && p.n != 32) return HQMQ_OK;
     // 8-byte vector loads of Q rows, table rows and sideband chunks; strides were checked by the caller
     if (p.n == 32) {
-        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, shmem, st, handled);
-        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, shmem, st, handled);
+        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, table_bytes, st, handled);
+        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, table_bytes, st, handled);
     }
-    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, shmem, st, handled);
-    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, shmem, st, handled);
+    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, table_bytes, st, handled);
+    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, table_bytes, st, handled);
 }
 
 }  // namespace hqmq

@@ -112,7 +112,7 @@ def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
     key = (tag, torch.device(device))
     buf = _WS.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        buf = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)   # attention counters start at zero
         _WS[key] = buf
     return buf
 

@@ -163,7 +163,7 @@ int hqmq_dequant_packed(const hqmq_packed *p, int dtype, int B, int H, int T, in
  * Query row i of sequence b sees key j iff j < kv_len[b] (T_kv when kv_len is
  * NULL) and (not causal or j <= i + causal_offset); causal_offset = 0 is the
  * reference's top-left alignment.
- *   workspace   hqmq_attn_workspace_bytes(...) bytes of scratch for split-KV partials */
+ *   workspace   hqmq_attn_workspace_bytes(...) bytes of scratch for split-KV partials, any content */
 typedef struct hqmq_attn_args {
     const void *Q; void *O;   /* D, [B][H_q][T_q][d_h]; strides in elements, last dim contiguous */
     int64_t q_sb, q_sh, q_st, o_sb, o_sh, o_st;
