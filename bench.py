@@ -27,6 +27,9 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the attention kernel from the FETCH_SIZE / WRITE_SIZE passes (scaled by a plain
+# 256 MiB copy), recorded in profiles/attn_fast_kernel_config2_32k_hbm_traffic.txt; known for these contexts only.
+MEASURED_TRAFFIC_BYTES = {32768: 37.83e6}
 
 
 def build_cache(q, T, dt, dev, seed):
@@ -105,6 +108,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of one HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--all-contexts", action="store_true", help="also report 4k / 8k / 16k")
+    ap.add_argument("--counters", action="store_true",
+                    help="for rocprofv3 --pmc runs: only 20 eager attention steps and 5 plain 256 MiB copies (the "
+                         "calibration kernel for FETCH_SIZE / WRITE_SIZE), no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: every box of this build has one, and the path needs no second "
@@ -146,6 +152,16 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.counters:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            step()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(f"counters mode: 20 attention steps of {cache_bytes} compressed bytes, 5 copies of {src.numel()} bytes")
+        return
     used_graph = False
     if not args.no_graph:
         try:
@@ -214,7 +230,7 @@ def main():
         "pct_of_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
         "max_abs_err_vs_dense_sdpa": max_err,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(T),
                      "kernel": "attn_fast_kernel<8,16,0,f16>", "kernel_us": round(us_main, 2),
                      "kernel_plus_combine_us": round(us_both, 2), "algorithmic_bytes_per_launch": cache_bytes},
         "quantize": {"GTok_per_s": round(gtok_s, 5), "us_per_call": round(us_quant, 1), "tokens": T,
