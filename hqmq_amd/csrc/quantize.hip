@@ -24,6 +24,9 @@
 
 namespace hqmq {
 
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
 constexpr int kQThreads = 256;
 constexpr int kSCap = 32;  // candidate secondaries kept per lane
 constexpr int kKCap = 24;  // candidate codewords kept per lane
@@ -117,7 +120,8 @@ __device__ __forceinline__ uint8_t gather_byte(const uint32_t *vals, int count, 
 template <class D, int ALGO>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
     using ST = typename D::storage;
-    extern __shared__ float sec[];  // [S][4]
+    extern __shared__ float sec[];  // [S][4] secondaries, then [S][4] fp16 columns of their rotation matrices
+    uint2 *rot = reinterpret_cast<uint2 *>(sec + 4 * a.S);
     __shared__ float radius_sh[kQThreads];
     __shared__ uint32_t code_sh[kQThreads];
     __shared__ uint32_t mask_sh[kQThreads];
@@ -133,6 +137,21 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
     const ST *jh = (const ST *)a.joint + (size_t)h * K * 4;
 
     for (int i = tid; i < S * 4; i += kQThreads) sec[i] = D::load(jh + i);  // rows k = s are q_s itself
+    if (ALGO == 0 && D::code != HQMQ_F32) {
+        // column i of M(q) with u * conj(q) = u M: (w,x,y,z), (-x,w,-z,y), (-y,z,w,-x), (-z,-y,x,w)
+        for (int i = tid; i < S * 4; i += kQThreads) {
+            const ST *q = jh + (i >> 2) * 4;
+            const float w = D::load(q), x = D::load(q + 1), y = D::load(q + 2), z = D::load(q + 3);
+            half4 c;
+            switch (i & 3) {
+                case 0: c = half4{(_Float16)w, (_Float16)x, (_Float16)y, (_Float16)z}; break;
+                case 1: c = half4{(_Float16)-x, (_Float16)w, (_Float16)-z, (_Float16)y}; break;
+                case 2: c = half4{(_Float16)-y, (_Float16)z, (_Float16)w, (_Float16)-x}; break;
+                default: c = half4{(_Float16)-z, (_Float16)-y, (_Float16)x, (_Float16)w}; break;
+            }
+            rot[i] = __builtin_bit_cast(uint2, c);
+        }
+    }
 
     float xv[4] = {0.f, 0.f, 0.f, 0.f};
     if (active) {
@@ -159,18 +178,37 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
         for (int j = 0; j < 4; j++) us[j] = search ? u[j] : (j == 0 ? 1.f : 0.f);
         const float ulen = sqrtf(fmaf(us[3], us[3], fmaf(us[2], us[2], fmaf(us[1], us[1], us[0] * us[0])))) * 1.000001f;
         const float E = ulen * (a.slack[h] + 1.01f * D::eps() + 9.5367e-7f);
-        const float margin2 = 4.f * E + ulen * 7.6294e-6f + 2.4e-7f;
+        const float margin2 = 4.f * E + ulen * 7.6294e-6f + 1.0e-6f;
         float m2 = -INFINITY;
         int cnt = 0;
-        for (int s = 0; s < S; s++) {
-            const float4 q = *reinterpret_cast<const float4 *>(sec + 4 * s);
-            float v[4];
-            rotate_conj(us, q.x, q.y, q.z, q.w, v);
-            const float b2 = best2_of(v);
-            m2 = fmaxf(m2, b2);
-            if (b2 >= m2 - margin2) {
-                if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
-                cnt++;
+        if (D::code != HQMQ_F32) {
+            // 16-bit dtypes: u and q_s are exact in fp16, so one v_mfma_f32_4x4x4_16B_f16 rotates the 64 chunks
+            // of the wavefront by q_s: block = 4 consecutive lanes, A = columns of the rotation matrix (the same
+            // for every block, lane i holds column i), B = the lane's own direction, D = its rotated chunk.
+            const half4 ub = half4{(_Float16)us[0], (_Float16)us[1], (_Float16)us[2], (_Float16)us[3]};
+            const uint2 *acol = rot + (tid & 3);
+            for (int s = 0; s < S; s++) {
+                const half4 am = __builtin_bit_cast(half4, acol[4 * s]);
+                const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                const float v[4] = {vv[0], vv[1], vv[2], vv[3]};
+                const float b2 = best2_of(v);
+                m2 = fmaxf(m2, b2);
+                if (b2 >= m2 - margin2) {
+                    if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
+                    cnt++;
+                }
+            }
+        } else {
+            for (int s = 0; s < S; s++) {
+                const float4 q = *reinterpret_cast<const float4 *>(sec + 4 * s);
+                float v[4];
+                rotate_conj(us, q.x, q.y, q.z, q.w, v);
+                const float b2 = best2_of(v);
+                m2 = fmaxf(m2, b2);
+                if (b2 >= m2 - margin2) {
+                    if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
+                    cnt++;
+                }
             }
         }
         if (search) {
@@ -183,12 +221,34 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
                     const float4 q = *reinterpret_cast<const float4 *>(sec + 4 * s);
                     float v[4];
                     rotate_conj(us, q.x, q.y, q.z, q.w, v);
-                    if (best2_of(v) < thr2) continue;  // entered while the running maximum was lower
+                    const float a0 = fabsf(v[0]), a1 = fabsf(v[1]), a2 = fabsf(v[2]), a3 = fabsf(v[3]);
+                    const float sum = (a0 + a1) + (a2 + a3);
+                    const float mx = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+                    if (fmaxf(mx + mx, sum) < thr2) continue;  // entered while the running maximum was lower
+                    // Usually exactly one Hurwitz unit of this secondary is inside the margin: the largest axis
+                    // or the all-signs-matched half unit. Count the others; only then enumerate all 24.
+                    const int n_axis = (a0 + a0 >= thr2) + (a1 + a1 >= thr2) + (a2 + a2 >= thr2) + (a3 + a3 >= thr2);
+                    const int n_flip = (sum - (a0 + a0) >= thr2) + (sum - (a1 + a1) >= thr2) + (sum - (a2 + a2) >= thr2) +
+                                       (sum - (a3 + a3) >= thr2);
+                    const int n_half = (sum >= thr2) + n_flip;
+                    if (n_axis + n_half == 1) {
+                        int pp;
+                        if (n_axis) {
+                            const int im = (a0 == mx) ? 0 : (a1 == mx) ? 1 : (a2 == mx) ? 2 : 3;
+                            const float vm = (a0 == mx) ? v[0] : (a1 == mx) ? v[1] : (a2 == mx) ? v[2] : v[3];
+                            pp = 2 * im + (vm < 0.f ? 1 : 0);
+                        } else {
+                            pp = 8 + ((v[0] < 0.f ? 8 : 0) | (v[1] < 0.f ? 4 : 0) | (v[2] < 0.f ? 2 : 0) | (v[3] < 0.f ? 1 : 0));
+                        }
+                        if (kcnt < kKCap) klist[kcnt][tid] = (uint16_t)(pp * S + s);
+                        kcnt++;
+                    } else {
 #pragma unroll
-                    for (int p = 0; p < 24; p++) {
-                        if (exact2_of(v, p) >= thr2) {
-                            if (kcnt < kKCap) klist[kcnt][tid] = (uint16_t)(p * S + s);
-                            kcnt++;
+                        for (int p = 0; p < 24; p++) {
+                            if (exact2_of(v, p) >= thr2) {
+                                if (kcnt < kKCap) klist[kcnt][tid] = (uint16_t)(p * S + s);
+                                kcnt++;
+                            }
                         }
                     }
                 }
@@ -265,7 +325,9 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
             if (a.main_plane) {
                 const int rb = (n * a.main_bits + 7) >> 3;
                 uint8_t *dst = a.main_plane + prow * rb;
-                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.main_bits, 0, byte);
+                if (a.main_bits == 16) reinterpret_cast<uint16_t *>(dst)[c] = (uint16_t)codes[c];   // one code per lane
+                else
+                    for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.main_bits, 0, byte);
             }
             if (a.aux_plane && a.aux_bits) {
                 const int rb = (n * a.aux_bits + 7) >> 3;
@@ -285,7 +347,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
 template <class D>
 static int launch_quantize(const QParams &p, int algo, hipStream_t st) {
     dim3 grid((p.T + p.tokens_per_block - 1) / p.tokens_per_block, p.B * p.H), block(kQThreads);
-    size_t shmem = (size_t)p.S * 4 * sizeof(float);
+    size_t shmem = (size_t)p.S * 4 * sizeof(float) + (size_t)p.S * 4 * sizeof(uint2);
     if (algo == 1) hipLaunchKernelGGL((quantize_kernel<D, 1>), grid, block, shmem, st, p);
     else hipLaunchKernelGGL((quantize_kernel<D, 0>), grid, block, shmem, st, p);
     return hip_status(hipGetLastError());
