@@ -1,18 +1,25 @@
 // Attention kernels specialised at compile time for the layouts the BASELINE shapes use:
 // d_h = 64 / 128, fp16 or bf16 caches, codes of 16+0 (s96_r4), 12+1 (s24_r3) or 16+3 (s192_r6) bits.
-// Same algorithm and lane mapping as the generic kernel in attention.hip (see the notes there); what
-// differs is that the dtype, the code widths and the aux width are template constants, the scales are
-// kept as raw 16-bit words until use, and the register budget is held to two wavefronts per SIMD so that
-// LDS gathers and MFMA latencies of one wavefront hide behind the other.
+//
+// Lane mapping (one wavefront, one 16-token tile): lane = 16 * grp + col decodes the CPL = d_h / 16 chunks
+// grp * CPL ... of token `col`, for K and for V alike.
+//   S^T = K . Q^T     v_mfma_f32_16x16x32_f16: A = two decoded K chunks of the lane, B = the matching Q chunks.
+//   V^T               the A operand of O^T = V^T . P^T needs 4 tokens of one d per lane, a decoded chunk is
+//                     4 d of one token.  The 16x16 transposition is one v_mfma_f32_16x16x16_f16 against the
+//                     identity (exact: every output is one fp16 input times 1.0) and two packed conversions,
+//                     instead of a dozen cross-lane VALU operations per chunk.
+//   O^T += V^T . P^T  v_mfma_f32_16x16x32_f16 over two tiles (32 tokens) at a time.
+// Row j of the V-side product is d = (grp * CPL + j) * 4 + e, the order the epilogue writes back.
+// Scores are kept as S^T * rs; 1/qmax is folded into the softmax scale and the epilogue.  Outlier chunks
+// (flag bit set) are zeroed in the decoded operand and enter through extra MFMAs with their verbatim values.
 #include "attention_common.h"
 
 namespace hqmq {
 
-template <int DT>
-__device__ __forceinline__ float cvt16(uint32_t bits16) {
-    if (DT == HQMQ_F16) return __half2float(__ushort_as_half((uint16_t)bits16));
-    return __uint_as_float(bits16 << 16);
-}
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef const uint2 __attribute__((address_space(3))) *lds_u2_ptr;
+
 template <int DT>
 __device__ __forceinline__ half4 chunk_to_half(uint2 w) {
     if (DT == HQMQ_F16) return __builtin_bit_cast(half4, w);
@@ -45,30 +52,29 @@ __device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, in
 
 constexpr int kFastWaves = 8;
 
-// codes, aux bits and raw 16-bit scales of one 64-token super-tile for one lane
-template <int NW, int AB>
+// codes, aux bits, raw 16-bit scales and flag words of one 64-token super-tile for one lane
+template <int NW, int AB, bool FLAGS>
 struct FastTile {
     uint32_t kw[4][NW], vw[4][NW];
     uint32_t kaux[AB ? 4 : 1], vaux[AB ? 4 : 1];
     uint2 ks[4], vs[4];
+    uint32_t kfl[FLAGS ? 4 : 1], vfl[FLAGS ? 4 : 1];   // flag bits of token `col` of tile u
+    int ksb[FLAGS ? 4 : 1], vsb[FLAGS ? 4 : 1];         // sideband slot of tile u's first flagged chunk
 };
 
 template <int NBYTES>
 __device__ __forceinline__ uint32_t load_small(const uint8_t *p) {
-    uint32_t v = 0;
+    if constexpr (NBYTES == 4) return *reinterpret_cast<const uint32_t *>(p);
+    else if constexpr (NBYTES == 2) return *reinterpret_cast<const uint16_t *>(p);
+    else {
+        uint32_t v = 0;
 #pragma unroll
-    for (int i = 0; i < NBYTES; i++) v |= (uint32_t)p[i] << (8 * i);
-    return v;
+        for (int i = 0; i < NBYTES; i++) v |= (uint32_t)p[i] << (8 * i);
+        return v;
+    }
 }
 
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-
-// two 16-bit scales (raw bits of dtype DT) as fp32 / as a packed fp16 pair
-template <int DT>
-__device__ __forceinline__ float scale_f32(uint32_t pair, int hi) {
-    if (DT == HQMQ_F16) return (float)__builtin_bit_cast(half2v, pair)[hi];
-    return __uint_as_float(hi ? (pair & 0xffff0000u) : (pair << 16));
-}
+// two 16-bit scales (raw bits of dtype DT) as a packed fp16 pair
 template <int DT>
 __device__ __forceinline__ half2v scale_h2(uint32_t pair) {
     if (DT == HQMQ_F16) return __builtin_bit_cast(half2v, pair);
@@ -77,29 +83,40 @@ __device__ __forceinline__ half2v scale_h2(uint32_t pair) {
     r[1] = (_Float16)__uint_as_float(pair & 0xffff0000u);
     return r;
 }
+// acc * scale[hi] (+ add): for fp16 scales one mixed-precision fma reads the half directly
+template <int DT>
+__device__ __forceinline__ float scaled(float acc, uint32_t pair, int hi, float add) {
+    if (DT == HQMQ_F16) return __builtin_fmaf(acc, (float)__builtin_bit_cast(half2v, pair)[hi], add);
+    return __builtin_fmaf(acc, __uint_as_float(hi ? (pair & 0xffff0000u) : (pair << 16)), add);
+}
 
-// The V table sits at a fixed LDS offset so that its gathers use the instruction's immediate offset.
+// The dynamic LDS block is the kernel's only LDS, so it starts at LDS address 0: the K table sits at byte 0,
+// the V table at kVTabOffset, and a gather addresses them with idx * 8 (+ the instruction's immediate offset).
 constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
 
-// Decodes the CPL chunks of one lane: gather from the LDS table (byte offset `tab`), times the radius code.
+template <int TAB_OFF>
+__device__ __forceinline__ half4 gather8(uint32_t byte_addr) {
+    return __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(byte_addr + TAB_OFF));
+}
+
+// Decodes the CPL chunks of one lane: gather from the LDS table, times the radius code.
 // 16+0 layout: the two radius codes of a dword become an fp16 pair with one shift, one and-or
-// (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract; the two table addresses take a
-// shift and a mask each.  IB = idx_bits when known at compile time (12 for s96), else 0.
-template <int CPL, int MB, int AB, int IB, int NW>
-__device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t aux, const char *tab, int idx_bits_rt,
-                                              half4 (&a)[CPL]) {
+// (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract.  IB = idx_bits when known at compile
+// time (12 for s96), else 0.
+template <int CPL, int MB, int AB, int IB, int NW, int TAB_OFF>
+__device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t aux, int idx_bits_rt, half4 (&a)[CPL]) {
     const int idx_bits = IB ? IB : idx_bits_rt;
     const uint32_t idx_mask = (1u << idx_bits) - 1u;
     if constexpr (MB == 16 && AB == 0) {
         const uint32_t rq2 = (0xffffu >> idx_bits) * 0x00010001u;
-        const uint2 *t2 = reinterpret_cast<const uint2 *>(tab);
+        const uint32_t im2 = idx_mask * 0x00010001u;
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
-            const uint32_t lo = w[i] & idx_mask, hi = (w[i] >> 16) & idx_mask;      // and / bit-field extract
+            const uint32_t ix = w[i] & im2;
             const uint32_t t = ((w[i] >> idx_bits) & rq2) | 0x64006400u;
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = __builtin_bit_cast(half4, t2[lo]) * r[0];
-            a[2 * i + 1] = __builtin_bit_cast(half4, t2[hi]) * r[1];
+            a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
+            a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
         }
     } else {
 #pragma unroll
@@ -107,9 +124,45 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
             uint32_t code = code_at<MB, NW>(w, j);
             if (AB) code |= ((aux >> (j * AB)) & ((1u << AB) - 1u)) << MB;
             const _Float16 rq = (_Float16)(uint16_t)(code >> idx_bits);
-            a[j] = __builtin_bit_cast(half4, reinterpret_cast<const uint2 *>(tab)[code & idx_mask]) * rq;
+            a[j] = gather8<TAB_OFF>((code & idx_mask) << 3) * rq;
         }
     }
+}
+
+__device__ __forceinline__ half8 cat8(half4 x, half4 y) { return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7); }
+
+// max over the four 16-lane rows (lanes l, l^16, l^32, l^48) without going through LDS
+__device__ __forceinline__ float row_max4(float x) {
+    const uint32_t b = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const float y = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const uint32_t c = __float_as_uint(y);
+    const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+__device__ __forceinline__ float row_sum4(float x) {
+    const uint32_t b = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const float y = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    const uint32_t c = __float_as_uint(y);
+    const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
+// inclusive prefix sum over the 16 lanes of a row (DPP row_shr with zero fill)
+__device__ __forceinline__ int row_prefix16(int x) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, true);
+    return x;
+}
+
+// fp32 4-vector (exact fp16 values) -> packed fp16
+__device__ __forceinline__ half4 pack4(float4v t) {
+    const auto lo = __builtin_amdgcn_cvt_pkrtz(t[0], t[1]);
+    const auto hi = __builtin_amdgcn_cvt_pkrtz(t[2], t[3]);
+    return __builtin_bit_cast(half4, uint2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)});
 }
 
 template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS>
@@ -118,14 +171,14 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     constexpr int NW = (NB + 3) / 4;
     constexpr int ABYTES = CPL * AB / 8;     // aux bytes per lane (CPL * AB is a multiple of 8 here)
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
+    static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = kFastWaves * 64;
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
-    const char *ktab_b = reinterpret_cast<const char *>(lds_tab), *vtab_b = ktab_b + kVTabOffset;
 
     const int bh = blockIdx.z, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
     const int cg = blockIdx.y, sp = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int G = p.G;
     constexpr int n = 4 * CPL, d_h = 16 * CPL;
     const int col = lane & 15, grp = lane >> 4;
@@ -145,53 +198,71 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
         lim_min = min(lim_min, __shfl_xor(lim_min, o));
     }
+    blk_lim = __builtin_amdgcn_readfirstlane(blk_lim);      // the same in every lane: all rows hold all 16 columns
+    lim_min = __builtin_amdgcn_readfirstlane(lim_min);
     int per_split = (blk_lim + p.n_splits - 1) / p.n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
     int per_wave = (b_end - b_begin + kFastWaves - 1) / kFastWaves;
     per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
+    // every super-tile starts at a multiple of 64 below T_kv <= t_cap (a multiple of 64): whole tiles are readable
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
 
     const size_t plane_row0 = (size_t)bh * p.t_cap;
     constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8, frb = (n + 7) / 8;
-    const int64_t tiles_cap = (p.t_cap + kTile - 1) / kTile;
+    const int64_t tiles_cap = p.t_cap / kTile;
     const int idx_bits = p.idx_bits;
-    const int v_tok = 4 * grp + (col & 3), v_grp = col >> 2;
     const uint16_t *ks_plane = (const uint16_t *)p.Kc.scale_plane + b * p.Kc.ssb + hkv * p.Kc.ssh;
     const uint16_t *vs_plane = (const uint16_t *)p.Vc.scale_plane + b * p.Vc.ssb + hkv * p.Vc.ssh;
-    const uint8_t *k_rows = p.Kc.main_plane + plane_row0 * mrb + grp * NB;
-    const uint8_t *v_rows = p.Vc.main_plane + plane_row0 * mrb + v_grp * NB;
-    const uint8_t *ka_rows = AB ? p.Kc.aux_plane + plane_row0 * arb + grp * ABYTES : nullptr;
-    const uint8_t *va_rows = AB ? p.Vc.aux_plane + plane_row0 * arb + v_grp * ABYTES : nullptr;
-    const int64_t last_row = p.t_cap - 1;
+    const uint8_t *k_rows = p.Kc.main_plane + plane_row0 * mrb;
+    const uint8_t *v_rows = p.Vc.main_plane + plane_row0 * mrb;
+    const uint8_t *ka_rows = AB ? p.Kc.aux_plane + plane_row0 * arb : nullptr;
+    const uint8_t *va_rows = AB ? p.Vc.aux_plane + plane_row0 * arb : nullptr;
+    const uint8_t *kf_rows = FLAGS ? p.Kc.flag_plane + plane_row0 * frb : nullptr;
+    const uint8_t *vf_rows = FLAGS ? p.Vc.flag_plane + plane_row0 * frb : nullptr;
+    const int32_t *k_toff = FLAGS ? p.Kc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
+    const int32_t *v_toff = FLAGS ? p.Vc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
+    const uint32_t main_off = (uint32_t)(col * mrb + grp * NB), aux_off = (uint32_t)(col * arb + grp * ABYTES);
+    const uint32_t flag_off = (uint32_t)(col * frb), scale_off = (uint32_t)(4 * grp);
 
-    auto load_super = [&](int t0, FastTile<NW, AB> &s) {
+    auto load_super = [&](int t0, FastTile<NW, AB, FLAGS> &s) {
+        const uint8_t *kb = k_rows + (size_t)t0 * mrb, *vb = v_rows + (size_t)t0 * mrb;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int64_t krow = min((int64_t)t0 + 16 * u + col, last_row);
-            const int64_t vrow = min((int64_t)t0 + 16 * u + v_tok, last_row);
-            load_bytes<NB>(k_rows + krow * mrb, s.kw[u]);
-            load_bytes<NB>(v_rows + vrow * mrb, s.vw[u]);
+            load_bytes<NB>(kb + main_off + u * 16 * mrb, s.kw[u]);
+            load_bytes<NB>(vb + main_off + u * 16 * mrb, s.vw[u]);
             if (AB) {
-                s.kaux[u] = load_small<ABYTES>(ka_rows + krow * arb);
-                s.vaux[u] = load_small<ABYTES>(va_rows + vrow * arb);
+                s.kaux[u] = load_small<ABYTES>(ka_rows + (size_t)t0 * arb + aux_off + u * 16 * arb);
+                s.vaux[u] = load_small<ABYTES>(va_rows + (size_t)t0 * arb + aux_off + u * 16 * arb);
             }
-            const int ts = t0 + 16 * u + 4 * grp;      // rows up to the plane capacity are readable
-            s.ks[u] = *reinterpret_cast<const uint2 *>(ks_plane + ts);
-            s.vs[u] = *reinterpret_cast<const uint2 *>(vs_plane + ts);
+            s.ks[u] = *reinterpret_cast<const uint2 *>(ks_plane + t0 + scale_off + 16 * u);
+            s.vs[u] = *reinterpret_cast<const uint2 *>(vs_plane + t0 + scale_off + 16 * u);
+            if (FLAGS) {
+                s.kfl[u] = load_small<frb>(kf_rows + (size_t)t0 * frb + flag_off + u * 16 * frb);
+                s.vfl[u] = load_small<frb>(vf_rows + (size_t)t0 * frb + flag_off + u * 16 * frb);
+                s.ksb[u] = k_toff[(t0 >> 4) + u];
+                s.vsb[u] = v_toff[(t0 >> 4) + u];
+            }
         }
     };
 
-    FastTile<NW, AB> cur;
+    FastTile<NW, AB, FLAGS> cur;
     if (t_begin < t_end) load_super(t_begin, cur);
 
-    half4 qf[CPL];
+    half8 qf[CPL / 2];
     {
         const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq * p.qsh + (int64_t)tq * p.qst + grp * CPL * 4;
 #pragma unroll
-        for (int j = 0; j < CPL; j++)
-            qf[j] = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 4 * j)) : half4{0, 0, 0, 0};
+        for (int j = 0; j < CPL / 2; j++) {
+            const half4 z = half4{0, 0, 0, 0};
+            const half4 lo = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
+            const half4 hi = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
+            qf[j] = cat8(lo, hi);
+        }
     }
+    half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
+#pragma unroll
+    for (int e = 0; e < 4; e++) ident[e] = (_Float16)((4 * grp + e) == col ? 1.f : 0.f);
 
     fill_tables16<DT, NT>(ktab, (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), p.Kc.K,
                           vtab, (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4), p.Vc.K);
@@ -203,44 +274,62 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     float4v acc[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
+    const half4 zero_h4 = half4{0, 0, 0, 0};
+    constexpr uint32_t cmask = (CPL >= 32) ? 0xffffffffu : ((1u << CPL) - 1u);
+    const int first = grp * CPL;
+
+    // Flag bookkeeping of one tile: the lane's CPL flag bits and the sideband slot of its first flagged chunk
+    // (tile offset + flagged chunks of earlier tokens of the tile + earlier chunks of the token).
+    auto lane_flags = [&](uint32_t fw, int tile_off, uint32_t &fl, int &slot) {
+        const int own = __popc(fw);
+        const int incl = row_prefix16(own);
+        fl = (fw >> first) & cmask;
+        slot = tile_off + incl - own + __popc(fw & ((1u << first) - 1u));
+    };
 
     for (int t0 = t_begin; t0 < t_end; t0 += kSuper) {
-        FastTile<NW, AB> nxt;
+        FastTile<NW, AB, FLAGS> nxt;
         const bool more = t0 + kSuper < t_end;
         if (more) load_super(t0 + kSuper, nxt);
 
         float4v sT[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            uint32_t fl = 0;
-            int sb_base = 0;
-            if (FLAGS)
-                tile_flags<CPL>(p.Kc, plane_row0, (int64_t)t0 + 16 * u, p.t_cap, frb,
-                                (size_t)bh * tiles_cap + min((int64_t)((t0 + 16 * u) >> 4), tiles_cap - 1), col, col, grp * CPL, fl, sb_base);
             half4 a[CPL];
-            decode_chunks<CPL, MB, AB, IB, NW>(cur.kw[u], AB ? cur.kaux[u] : 0u, ktab_b, idx_bits, a);
-            float4v s = float4v{0.f, 0.f, 0.f, 0.f}, so = float4v{0.f, 0.f, 0.f, 0.f};
+            decode_chunks<CPL, MB, AB, IB, NW, 0>(cur.kw[u], AB ? cur.kaux[u] : 0u, idx_bits, a);
+            float4v s = zero4, so = zero4;
+            if (FLAGS) {
+                const uint32_t fw = cur.kfl[u];
+                if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
+                    uint32_t fl;
+                    int slot;
+                    lane_flags(fw, cur.ksb[u], fl, slot);
 #pragma unroll
-            for (int j = 0; j < CPL; j++) {
-                if (FLAGS) {
-                    const bool f = (fl >> j) & 1u;
-                    if (__builtin_amdgcn_ballot_w64(f) != 0) {
-                        half4 ao = half4{0, 0, 0, 0};
-                        if (f) {
-                            ao = outlier_chunk(p.Kc, DT, bh, sb_base + __popc(fl & ((1u << j) - 1u)));
-                            a[j] = half4{0, 0, 0, 0};
+                    for (int j = 0; j < CPL; j++)
+                        if ((fl >> j) & 1u) a[j] = zero_h4;
+                    uint32_t rem = fl;
+                    while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
+                        const bool has = rem != 0;
+                        const int jme = has ? __builtin_ctz(rem) : 255;
+                        const half4 val = has ? outlier_chunk(p.Kc, DT, bh, slot) : zero_h4;
+                        slot++;
+                        rem &= rem - 1u;
+#pragma unroll
+                        for (int jj = 0; jj < CPL / 2; jj++) {
+                            const bool m0 = jme == 2 * jj, m1 = jme == 2 * jj + 1;
+                            if (__builtin_amdgcn_ballot_w64(m0 || m1) != 0)
+                                so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(m0 ? val : zero_h4, m1 ? val : zero_h4), qf[jj], so, 0, 0, 0);
                         }
-                        so = __builtin_amdgcn_mfma_f32_16x16x16f16(ao, qf[j], so, 0, 0, 0);
                     }
                 }
-                s = __builtin_amdgcn_mfma_f32_16x16x16f16(a[j], qf[j], s, 0, 0, 0);
             }
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float rs = scale_f32<DT>(e < 2 ? cur.ks[u].x : cur.ks[u].y, e & 1);
-                s[e] = s[e] * rs;
-                if (FLAGS) s[e] = fmaf(so[e], qmaxf, s[e]);
-            }
+            for (int jj = 0; jj < CPL / 2; jj++)
+                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                s[e] = scaled<DT>(s[e], e < 2 ? cur.ks[u].x : cur.ks[u].y, e & 1, FLAGS ? so[e] * qmaxf : 0.f);
             sT[u] = s;
         }
         // ---- mask (boundary super-tiles only), online softmax ----
@@ -257,8 +346,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
                            fmaxf(fmaxf(sT[1][0], sT[1][1]), fmaxf(sT[1][2], sT[1][3])));
         tmax = fmaxf(tmax, fmaxf(fmaxf(fmaxf(sT[2][0], sT[2][1]), fmaxf(sT[2][2], sT[2][3])),
                                  fmaxf(fmaxf(sT[3][0], sT[3][1]), fmaxf(sT[3][2], sT[3][3]))));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        tmax = row_max4(tmax);
         const float m_new = fmaxf(m_run, tmax);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {     // rescale only when some column's maximum moved
@@ -283,43 +371,55 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
             if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
         }
-        // ---- O^T += V^T . P^T (the 1/qmax of the radius is applied once, in the epilogue) ----
+        // ---- O^T += V^T . P^T, two tiles per MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            uint32_t fl = 0;
-            int sb_base = 0;
-            if (FLAGS)
-                tile_flags<CPL>(p.Vc, plane_row0, (int64_t)t0 + 16 * u, p.t_cap, frb,
-                                (size_t)bh * tiles_cap + min((int64_t)((t0 + 16 * u) >> 4), tiles_cap - 1), col, v_tok, v_grp * CPL, fl, sb_base);
-            half4 a[CPL];
-            decode_chunks<CPL, MB, AB, IB, NW>(cur.vw[u], AB ? cur.vaux[u] : 0u, vtab_b, idx_bits, a);
+        for (int up = 0; up < 2; up++) {
+            half4 av[2][CPL];
 #pragma unroll
-            for (int j = 0; j < CPL; j++) {
+            for (int h = 0; h < 2; h++) {
+                const int u = 2 * up + h;
+                decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(cur.vw[u], AB ? cur.vaux[u] : 0u, idx_bits, av[h]);
                 if (FLAGS) {
-                    const bool f = (fl >> j) & 1u;
-                    if (__builtin_amdgcn_ballot_w64(f) != 0) {
-                        half4 ao = half4{0, 0, 0, 0};
-                        if (f) {
-                            ao = outlier_chunk(p.Vc, DT, bh, sb_base + __popc(fl & ((1u << j) - 1u)));
-                            a[j] = half4{0, 0, 0, 0};
+                    const uint32_t fw = cur.vfl[u];
+                    if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
+                        uint32_t fl;
+                        int slot;
+                        lane_flags(fw, cur.vsb[u], fl, slot);
+#pragma unroll
+                        for (int j = 0; j < CPL; j++)
+                            if ((fl >> j) & 1u) av[h][j] = zero_h4;
+                        uint32_t rem = fl;
+                        while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
+                            const bool has = rem != 0;
+                            const int jme = has ? __builtin_ctz(rem) : 255;
+                            const half4 val = has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4;
+                            slot++;
+                            rem &= rem - 1u;
+#pragma unroll
+                            for (int j = 0; j < CPL; j++) {
+                                const bool mj = jme == j;
+                                if (__builtin_amdgcn_ballot_w64(mj) != 0) {
+                                    const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
+                                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo[u], acc[j], 0, 0, 0);
+                                }
+                            }
                         }
-                        uint2 ro = __builtin_bit_cast(uint2, ao);
-                        quad_transpose(ro.x, ro.y, lane);
-                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, ro), pTo[u], acc[j], 0, 0, 0);
                     }
                 }
-                uint2 r = __builtin_bit_cast(uint2, a[j]);
-                quad_transpose(r.x, r.y, lane);
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, r), pT[u], acc[j], 0, 0, 0);
+            }
+            const half8 pp = cat8(pT[2 * up], pT[2 * up + 1]);
+#pragma unroll
+            for (int j = 0; j < CPL; j++) {
+                const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
+                const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
             }
         }
         if (more) cur = nxt;
     }
 
     // ---- merge the block's waves through LDS ----
-    float l_tot = l_run;
-    l_tot += __shfl_xor(l_tot, 16);
-    l_tot += __shfl_xor(l_tot, 32);
+    const float l_tot = row_sum4(l_run);
     float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][d_h + 2]
     __syncthreads();
     {
@@ -362,9 +462,8 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
 }
 
 template <int CPL, int MB, int AB, int IB, int DT>
-static int launch_one(const AttnParams &p, bool flags, dim3 grid, size_t table_bytes, hipStream_t st) {
+static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
-    (void)table_bytes;
     size_t shmem = (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 2) * sizeof(float);
     if (shmem < merge) shmem = merge;
@@ -378,28 +477,33 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, size_t table_b
 }
 
 template <int CPL, int DT>
-static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled) {
+static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
     *handled = true;
-    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, table_bytes, st);
-    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, table_bytes, st);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, table_bytes, st);
-    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, table_bytes, st);
+    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st);
+    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st);
     *handled = false;
     return HQMQ_OK;
 }
 
 int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled) {
+    (void)table_bytes;
     *handled = false;
     if (p.dtype != HQMQ_F16 && p.dtype != HQMQ_BF16) return HQMQ_OK;
     if (p.n != 16 && p.n != 32) return HQMQ_OK;
+    if (p.t_cap % kSuper) return HQMQ_OK;
+    // vector loads of plane rows: main rows 16-byte aligned (checked by the caller), aux and flag rows to their width
+    if (p.aux_bits && (((uintptr_t)p.Kc.aux_plane | (uintptr_t)p.Vc.aux_plane) & 3)) return HQMQ_OK;
+    if (flags && (((uintptr_t)p.Kc.flag_plane | (uintptr_t)p.Vc.flag_plane) & 3)) return HQMQ_OK;
     // 8-byte vector loads of Q rows, table rows and sideband chunks; strides were checked by the caller
     if (p.n == 32) {
-        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, table_bytes, st, handled);
-        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, table_bytes, st, handled);
+        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, st, handled);
+        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, st, handled);
     }
-    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, table_bytes, st, handled);
-    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, table_bytes, st, handled);
+    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, st, handled);
+    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, st, handled);
 }
 
 }  // namespace hqmq
