@@ -52,14 +52,19 @@ __device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, in
 
 constexpr int kFastWaves = 8;
 
-// codes, aux bits, raw 16-bit scales and flag words of one 64-token super-tile for one lane
+// codes, aux bits, raw 16-bit scales and flag words of 32 tokens (two 16-token tiles) for one lane
 template <int NW, int AB, bool FLAGS>
+struct HalfTile {
+    uint32_t kw[2][NW], vw[2][NW];
+    uint32_t kaux[AB ? 2 : 1], vaux[AB ? 2 : 1];
+    uint2 ks[2], vs[2];
+    uint32_t kfl[FLAGS ? 2 : 1], vfl[FLAGS ? 2 : 1];   // flag bits of token `col` of tile u
+    int ksb[FLAGS ? 2 : 1], vsb[FLAGS ? 2 : 1];         // sideband slot of tile u's first flagged chunk
+};
+// the unit of prefetch: NH half-tiles (64 tokens; 32 for the variants with outlier flags, which need the registers)
+template <int NW, int AB, bool FLAGS, int NH>
 struct FastTile {
-    uint32_t kw[4][NW], vw[4][NW];
-    uint32_t kaux[AB ? 4 : 1], vaux[AB ? 4 : 1];
-    uint2 ks[4], vs[4];
-    uint32_t kfl[FLAGS ? 4 : 1], vfl[FLAGS ? 4 : 1];   // flag bits of token `col` of tile u
-    int ksb[FLAGS ? 4 : 1], vsb[FLAGS ? 4 : 1];         // sideband slot of tile u's first flagged chunk
+    HalfTile<NW, AB, FLAGS> h[NH];
 };
 
 template <int NBYTES>
@@ -173,6 +178,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = kFastWaves * 64;
+    constexpr int NH = FLAGS ? 1 : 2, STEP = 32 * NH;
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
 
@@ -225,29 +231,35 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const uint32_t main_off = (uint32_t)(col * mrb + grp * NB), aux_off = (uint32_t)(col * arb + grp * ABYTES);
     const uint32_t flag_off = (uint32_t)(col * frb), scale_off = (uint32_t)(4 * grp);
 
-    auto load_super = [&](int t0, FastTile<NW, AB, FLAGS> &s) {
-        const uint8_t *kb = k_rows + (size_t)t0 * mrb, *vb = v_rows + (size_t)t0 * mrb;
+    auto load_super = [&](int t0, FastTile<NW, AB, FLAGS, NH> &s) {
+        // in the order the half-steps consume them: K, then V, of tokens 0..31, then the same of tokens 32..63
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            load_bytes<NB>(kb + main_off + u * 16 * mrb, s.kw[u]);
-            load_bytes<NB>(vb + main_off + u * 16 * mrb, s.vw[u]);
-            if (AB) {
-                s.kaux[u] = load_small<ABYTES>(ka_rows + (size_t)t0 * arb + aux_off + u * 16 * arb);
-                s.vaux[u] = load_small<ABYTES>(va_rows + (size_t)t0 * arb + aux_off + u * 16 * arb);
+        for (int hh = 0; hh < NH; hh++) {
+            const int th = t0 + 32 * hh;
+            const uint8_t *kb = k_rows + (size_t)th * mrb, *vb = v_rows + (size_t)th * mrb;
+            HalfTile<NW, AB, FLAGS> &h = s.h[hh];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                load_bytes<NB>(kb + main_off + u * 16 * mrb, h.kw[u]);
+                if (AB) h.kaux[u] = load_small<ABYTES>(ka_rows + (size_t)th * arb + aux_off + u * 16 * arb);
+                if (FLAGS) {
+                    h.kfl[u] = load_small<frb>(kf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
+                    h.ksb[u] = k_toff[(th >> 4) + u];
+                }
+                h.ks[u] = *reinterpret_cast<const uint2 *>(ks_plane + th + scale_off + 16 * u);
             }
-            s.ks[u] = *reinterpret_cast<const uint2 *>(ks_plane + t0 + scale_off + 16 * u);
-            s.vs[u] = *reinterpret_cast<const uint2 *>(vs_plane + t0 + scale_off + 16 * u);
-            if (FLAGS) {
-                s.kfl[u] = load_small<frb>(kf_rows + (size_t)t0 * frb + flag_off + u * 16 * frb);
-                s.vfl[u] = load_small<frb>(vf_rows + (size_t)t0 * frb + flag_off + u * 16 * frb);
-                s.ksb[u] = k_toff[(t0 >> 4) + u];
-                s.vsb[u] = v_toff[(t0 >> 4) + u];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                load_bytes<NB>(vb + main_off + u * 16 * mrb, h.vw[u]);
+                if (AB) h.vaux[u] = load_small<ABYTES>(va_rows + (size_t)th * arb + aux_off + u * 16 * arb);
+                if (FLAGS) {
+                    h.vfl[u] = load_small<frb>(vf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
+                    h.vsb[u] = v_toff[(th >> 4) + u];
+                }
+                h.vs[u] = *reinterpret_cast<const uint2 *>(vs_plane + th + scale_off + 16 * u);
             }
         }
     };
-
-    FastTile<NW, AB, FLAGS> cur;
-    if (t_begin < t_end) load_super(t_begin, cur);
 
     half8 qf[CPL / 2];
     {
@@ -260,12 +272,35 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             qf[j] = cat8(lo, hi);
         }
     }
+    // First batch of codeword-table loads (the longest dependency chain of the prologue: load, convert, LDS
+    // store, barrier), then the wavefront's first super-tile; the LDS stores follow.  The Q rows were requested
+    // before both so that waiting for them does not wait for the tiles.
+    constexpr int FU = 5;
+    const uint2 *ksrc = (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), *vsrc = (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4);
+    const int Kk = p.Kc.K, Kv = p.Vc.K;
+    uint2 tk[FU], tv[FU];
+#pragma unroll
+    for (int u = 0; u < FU; u++) {
+        const int k = threadIdx.x + u * NT;
+        tk[u] = k < Kk ? ksrc[k] : uint2{0, 0};
+        tv[u] = k < Kv ? vsrc[k] : uint2{0, 0};
+    }
+
+    FastTile<NW, AB, FLAGS, NH> cur;
+    if (t_begin < t_end) load_super(t_begin, cur);
+
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
     for (int e = 0; e < 4; e++) ident[e] = (_Float16)((4 * grp + e) == col ? 1.f : 0.f);
 
-    fill_tables16<DT, NT>(ktab, (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), p.Kc.K,
-                          vtab, (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4), p.Vc.K);
+#pragma unroll
+    for (int u = 0; u < FU; u++) {
+        const int k = threadIdx.x + u * NT;
+        if (k < Kk) ktab[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tk[u]));
+        if (k < Kv) vtab[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tv[u]));
+    }
+    if (max(Kk, Kv) > FU * NT)
+        fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
     __syncthreads();
 
     // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
@@ -288,23 +323,20 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         slot = tile_off + incl - own + __popc(fw & ((1u << first) - 1u));
     };
 
-    for (int t0 = t_begin; t0 < t_end; t0 += kSuper) {
-        FastTile<NW, AB, FLAGS> nxt;
-        const bool more = t0 + kSuper < t_end;
-        if (more) load_super(t0 + kSuper, nxt);
-
-        float4v sT[4];
+    // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.
+    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th) {
+        float4v sT[2];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < 2; u++) {
             half4 a[CPL];
-            decode_chunks<CPL, MB, AB, IB, NW, 0>(cur.kw[u], AB ? cur.kaux[u] : 0u, idx_bits, a);
+            decode_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, a);
             float4v s = zero4, so = zero4;
             if (FLAGS) {
-                const uint32_t fw = cur.kfl[u];
+                const uint32_t fw = h.kfl[u];
                 if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
                     uint32_t fl;
                     int slot;
-                    lane_flags(fw, cur.ksb[u], fl, slot);
+                    lane_flags(fw, h.ksb[u], fl, slot);
 #pragma unroll
                     for (int j = 0; j < CPL; j++)
                         if ((fl >> j) & 1u) a[j] = zero_h4;
@@ -329,23 +361,21 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
                 s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                s[e] = scaled<DT>(s[e], e < 2 ? cur.ks[u].x : cur.ks[u].y, e & 1, FLAGS ? so[e] * qmaxf : 0.f);
+                s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[e] * qmaxf : 0.f);
             sT[u] = s;
         }
-        // ---- mask (boundary super-tiles only), online softmax ----
-        if (!(t0 + kSuper <= lim_min && t0 + kSuper <= t_end)) {
+        // ---- mask (boundary half-steps only), online softmax ----
+        if (!(th + 32 <= lim_min && th + 32 <= t_end)) {
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < 2; u++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const int t = t0 + 16 * u + 4 * grp + e;
+                    const int t = th + 16 * u + 4 * grp + e;
                     if (!(t < col_lim && t < t_end)) sT[u][e] = -INFINITY;
                 }
         }
         float tmax = fmaxf(fmaxf(fmaxf(sT[0][0], sT[0][1]), fmaxf(sT[0][2], sT[0][3])),
                            fmaxf(fmaxf(sT[1][0], sT[1][1]), fmaxf(sT[1][2], sT[1][3])));
-        tmax = fmaxf(tmax, fmaxf(fmaxf(fmaxf(sT[2][0], sT[2][1]), fmaxf(sT[2][2], sT[2][3])),
-                                 fmaxf(fmaxf(sT[3][0], sT[3][1]), fmaxf(sT[3][2], sT[3][3]))));
         tmax = row_max4(tmax);
         const float m_new = fmaxf(m_run, tmax);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -357,78 +387,81 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             m_run = m_new;
         }
         const float mc = -m_use * c;
-        half4 pT[4], pTo[4];
+        half4 pT[2], pTo[2];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < 2; u++) {
             float pe[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[u][e], c, mc));
                 l_run += pe[e];
             }
-            const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(cur.vs[u].x);
-            const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(cur.vs[u].y);
+            const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(h.vs[u].x);
+            const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(h.vs[u].y);
             pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
             if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
         }
-        // ---- O^T += V^T . P^T, two tiles per MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
+        // ---- O^T += V^T . P^T, both tiles in one MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
+        half4 av[2][CPL];
 #pragma unroll
-        for (int up = 0; up < 2; up++) {
-            half4 av[2][CPL];
+        for (int u = 0; u < 2; u++) {
+            decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, av[u]);
+            if (FLAGS) {
+                const uint32_t fw = h.vfl[u];
+                if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
+                    uint32_t fl;
+                    int slot;
+                    lane_flags(fw, h.vsb[u], fl, slot);
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int u = 2 * up + h;
-                decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(cur.vw[u], AB ? cur.vaux[u] : 0u, idx_bits, av[h]);
-                if (FLAGS) {
-                    const uint32_t fw = cur.vfl[u];
-                    if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
-                        uint32_t fl;
-                        int slot;
-                        lane_flags(fw, cur.vsb[u], fl, slot);
+                    for (int j = 0; j < CPL; j++)
+                        if ((fl >> j) & 1u) av[u][j] = zero_h4;
+                    uint32_t rem = fl;
+                    while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
+                        const bool has = rem != 0;
+                        const int jme = has ? __builtin_ctz(rem) : 255;
+                        const half4 val = has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4;
+                        slot++;
+                        rem &= rem - 1u;
 #pragma unroll
-                        for (int j = 0; j < CPL; j++)
-                            if ((fl >> j) & 1u) av[h][j] = zero_h4;
-                        uint32_t rem = fl;
-                        while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
-                            const bool has = rem != 0;
-                            const int jme = has ? __builtin_ctz(rem) : 255;
-                            const half4 val = has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4;
-                            slot++;
-                            rem &= rem - 1u;
-#pragma unroll
-                            for (int j = 0; j < CPL; j++) {
-                                const bool mj = jme == j;
-                                if (__builtin_amdgcn_ballot_w64(mj) != 0) {
-                                    const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
-                                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo[u], acc[j], 0, 0, 0);
-                                }
+                        for (int j = 0; j < CPL; j++) {
+                            const bool mj = jme == j;
+                            if (__builtin_amdgcn_ballot_w64(mj) != 0) {
+                                const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
+                                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo[u], acc[j], 0, 0, 0);
                             }
                         }
                     }
                 }
             }
-            const half8 pp = cat8(pT[2 * up], pT[2 * up + 1]);
-#pragma unroll
-            for (int j = 0; j < CPL; j++) {
-                const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
-                const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
-            }
         }
+        const half8 pp = cat8(pT[0], pT[1]);
+#pragma unroll
+        for (int j = 0; j < CPL; j++) {
+            const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
+            const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
+        }
+    };
+
+    for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
+        FastTile<NW, AB, FLAGS, NH> nxt;
+        const bool more = t0 + STEP < t_end;
+        if (more) load_super(t0 + STEP, nxt);
+        half_step(cur.h[0], t0);
+        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32);
         if (more) cur = nxt;
     }
 
-    // ---- merge the block's waves through LDS ----
+    // ---- merge the block's waves through LDS: rows of [d_h accumulators, m, l, pad] ----
+    constexpr int RS = d_h + 4;
     const float l_tot = row_sum4(l_run);
-    float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][d_h + 2]
+    float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][RS]
     __syncthreads();
     {
-        float *wp = red + ((size_t)wave * 16 + col) * (d_h + 2);
-        if (grp == 0) { wp[0] = m_run; wp[1] = l_tot; }
+        float *wp = red + ((size_t)wave * 16 + col) * RS;
+        if (grp == 0) { wp[d_h] = m_run; wp[d_h + 1] = l_tot; }
 #pragma unroll
-        for (int j = 0; j < CPL; j++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) wp[2 + grp * CPL * 4 + 4 * j + e] = acc[j][e];
+        for (int j = 0; j < CPL; j++) *reinterpret_cast<float4v *>(wp + grp * CPL * 4 + 4 * j) = acc[j];
     }
     __syncthreads();
     const int ncols = min(16, p.Tq * G - cg * 16);
@@ -438,15 +471,15 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         const int ci = cg * 16 + cc;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kFastWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * (d_h + 2)]);
+        for (int w = 0; w < kFastWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
         float l = 0.f, a = 0.f;
         if (m > -INFINITY) {
 #pragma unroll
             for (int w = 0; w < kFastWaves; w++) {
-                const float *q = red + ((size_t)w * 16 + cc) * (d_h + 2);
-                const float f = __builtin_amdgcn_exp2f((q[0] - m) * c);
-                l = fmaf(q[1], f, l);
-                a = fmaf(q[2 + e], f, a);
+                const float *q = red + ((size_t)w * 16 + cc) * RS;
+                const float f = __builtin_amdgcn_exp2f((q[d_h] - m) * c);
+                l = fmaf(q[d_h + 1], f, l);
+                a = fmaf(q[e], f, a);
             }
         }
         const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
@@ -465,7 +498,7 @@ template <int CPL, int MB, int AB, int IB, int DT>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
     size_t shmem = (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
-    const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 2) * sizeof(float);
+    const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 4) * sizeof(float);
     if (shmem < merge) shmem = merge;
     auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true> : attn_fast_kernel<CPL, MB, AB, IB, DT, false>;
     if (shmem > 48 * 1024) {
