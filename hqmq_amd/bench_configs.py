@@ -124,7 +124,7 @@ def run(cfg, steps):
             valid = torch.arange(pt.t_cap, device=DEV).view(1, 1, -1) < lens_dev.view(B, 1, 1)
             flagged += int((bits * valid).sum())
     step_bytes = 2 * Hkv * tokens * row + flagged * 4 * cache.K.scale.element_size()
-    n_splits = ops.pick_splits(B, Hq, Hkv, 1, T if lens is None else int(lens.max()))
+    n_splits = ops.pick_splits(B, Hq, Hkv, 1, T if lens is None else int(lens.max()), lens is not None)
 
     def attend():
         hqmq.fused_attention_packed(Q, cache, kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out)

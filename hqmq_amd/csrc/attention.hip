@@ -379,11 +379,13 @@ extern "C" int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, i
 
 // Blocks per (sequence, KV head, column group): one block per CU, each of a block's eight wavefronts
 // keeping at least one 64-token super-tile.
-extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv) {
+extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv, int ragged) {
     if (B < 1 || H_q < 1 || H_kv < 1 || T_q < 1 || T_kv < 1) return 1;
     const int G = H_q / H_kv;
     const int64_t base = (int64_t)B * H_kv * ((T_q * G + 15) / 16);
-    int64_t s = (256 + base - 1) / base;
+    // sequences of different lengths: four rounds of smaller blocks even out the finishing times
+    const int64_t target = ragged ? 1024 : 256;
+    int64_t s = (target + base - 1) / base;
     const int64_t cap = (T_kv + 8 * kSuper - 1) / (8 * kSuper);
     if (s > cap) s = cap;
     if (s < 1) s = 1;
@@ -429,7 +431,7 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if (((uintptr_t)a->K.main_plane & 15) || ((uintptr_t)a->V.main_plane & 15)) return HQMQ_ERR_ALIGN;
     if (flags && (((uintptr_t)a->K.sideband % (4 * elt)) || ((uintptr_t)a->V.sideband % (4 * elt)))) return HQMQ_ERR_ALIGN;
 
-    int n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv);
+    int n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv, a->kv_len != nullptr);
     if (n_splits > 8192) return HQMQ_ERR_SHAPE;   // the merge keeps one weight per split in LDS
     if (n_splits > 1) {
         if (!a->workspace) return HQMQ_ERR_NULL;

@@ -52,14 +52,18 @@ __device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, in
 
 constexpr int kFastWaves = 8;
 
-// codes, aux bits, raw 16-bit scales and flag words of 32 tokens (two 16-token tiles) for one lane
+// codes, aux bits and raw 16-bit scales of 32 tokens (two 16-token tiles) for one lane
 template <int NW, int AB, bool FLAGS>
 struct HalfTile {
     uint32_t kw[2][NW], vw[2][NW];
     uint32_t kaux[AB ? 2 : 1], vaux[AB ? 2 : 1];
     uint2 ks[2], vs[2];
-    uint32_t kfl[FLAGS ? 2 : 1], vfl[FLAGS ? 2 : 1];   // flag bits of token `col` of tile u
-    int ksb[FLAGS ? 2 : 1], vsb[FLAGS ? 2 : 1];         // sideband slot of tile u's first flagged chunk
+};
+// flag words of the same 32 tokens; they travel one half-step ahead of the codes, so that the sideband chunks
+// they point to can be requested a whole half-step before use
+struct FlagTile {
+    uint32_t kfl[2], vfl[2];   // flag bits of token `col` of tile u
+    int ksb[2], vsb[2];        // sideband slot of tile u's first flagged chunk
 };
 // the unit of prefetch: NH half-tiles (64 tokens; 32 for the variants with outlier flags, which need the registers)
 template <int NW, int AB, bool FLAGS, int NH>
@@ -242,20 +246,12 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             for (int u = 0; u < 2; u++) {
                 load_bytes<NB>(kb + main_off + u * 16 * mrb, h.kw[u]);
                 if (AB) h.kaux[u] = load_small<ABYTES>(ka_rows + (size_t)th * arb + aux_off + u * 16 * arb);
-                if (FLAGS) {
-                    h.kfl[u] = load_small<frb>(kf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
-                    h.ksb[u] = k_toff[(th >> 4) + u];
-                }
                 h.ks[u] = *reinterpret_cast<const uint2 *>(ks_plane + th + scale_off + 16 * u);
             }
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 load_bytes<NB>(vb + main_off + u * 16 * mrb, h.vw[u]);
                 if (AB) h.vaux[u] = load_small<ABYTES>(va_rows + (size_t)th * arb + aux_off + u * 16 * arb);
-                if (FLAGS) {
-                    h.vfl[u] = load_small<frb>(vf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
-                    h.vsb[u] = v_toff[(th >> 4) + u];
-                }
                 h.vs[u] = *reinterpret_cast<const uint2 *>(vs_plane + th + scale_off + 16 * u);
             }
         }
@@ -272,6 +268,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             qf[j] = cat8(lo, hi);
         }
     }
+    auto load_flags = [&](int th, FlagTile &f) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            f.kfl[u] = load_small<frb>(kf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
+            f.vfl[u] = load_small<frb>(vf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
+            f.ksb[u] = k_toff[(th >> 4) + u];
+            f.vsb[u] = v_toff[(th >> 4) + u];
+        }
+    };
+
     // First batch of codeword-table loads (the longest dependency chain of the prologue: load, convert, LDS
     // store, barrier), then the wavefront's first super-tile; the LDS stores follow.  The Q rows were requested
     // before both so that waiting for them does not wait for the tiles.
@@ -287,7 +293,12 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
 
     FastTile<NW, AB, FLAGS, NH> cur;
-    if (t_begin < t_end) load_super(t_begin, cur);
+    FlagTile f0 = {}, f1 = {};
+    if (t_begin < t_end) {
+        if (FLAGS) load_flags(t_begin, f0);
+        load_super(t_begin, cur);
+        if (FLAGS && t_begin + STEP < t_end) load_flags(t_begin + STEP, f1);
+    }
 
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
@@ -323,42 +334,94 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         slot = tile_off + incl - own + __popc(fw & ((1u << first) - 1u));
     };
 
-    // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.
-    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th) {
+    // Outlier chunks of one tile: flag bookkeeping done and the lane's first two sideband chunks requested.
+    struct OutPre {
+        bool any;           // some lane of the wavefront has a flagged chunk in this tile
+        uint32_t fl;        // the lane's CPL flag bits
+        int slot;           // sideband slot of its first flagged chunk
+        half4 v0, v1;       // its first two flagged chunks (requested early; more are rare and loaded on demand)
+    };
+    auto out_issue = [&](const PackedDev &pc, uint32_t fw, int tile_off, OutPre &o) {
+        o.any = __builtin_amdgcn_ballot_w64(fw != 0) != 0;
+        o.fl = 0;
+        o.slot = 0;
+        o.v0 = zero_h4;
+        o.v1 = zero_h4;
+        if (o.any) {
+            lane_flags(fw, tile_off, o.fl, o.slot);
+            const uint32_t r1 = o.fl & (o.fl - 1u);
+            if (o.fl) o.v0 = outlier_chunk(pc, DT, bh, o.slot);
+            if (r1) o.v1 = outlier_chunk(pc, DT, bh, o.slot + 1);
+        }
+    };
+    // Calls use(j, value) for every flagged chunk of the lane, j wave-uniform per call... the callee masks by lane.
+    // K side: the verbatim chunks times Q, accumulated unscaled in `so`.
+    auto out_apply_k = [&](const OutPre &o, float4v &so) {
+        if (!o.any) return;
+        auto one = [&](int jme, half4 val) {
+#pragma unroll
+            for (int jj = 0; jj < CPL / 2; jj++) {
+                const bool m0 = jme == 2 * jj, m1 = jme == 2 * jj + 1;
+                if (__builtin_amdgcn_ballot_w64(m0 || m1) != 0)
+                    so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(m0 ? val : zero_h4, m1 ? val : zero_h4), qf[jj], so, 0, 0, 0);
+            }
+        };
+        one(o.fl ? __builtin_ctz(o.fl) : 255, o.v0);
+        const uint32_t r1 = o.fl & (o.fl - 1u);
+        if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
+            one(r1 ? __builtin_ctz(r1) : 255, o.v1);
+            uint32_t rem = r1 & (r1 - 1u);
+            int slot = o.slot + 2;
+            while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
+                const bool has = rem != 0;
+                one(has ? __builtin_ctz(rem) : 255, has ? outlier_chunk(p.Kc, DT, bh, slot) : zero_h4);
+                slot++;
+                rem &= rem - 1u;
+            }
+        }
+    };
+    // V side: the verbatim chunks, transposed, times the unscaled probabilities of the tile.
+    auto out_apply_v = [&](const OutPre &o, half4 pTo) {
+        if (!o.any) return;
+        auto one = [&](int jme, half4 val) {
+#pragma unroll
+            for (int j = 0; j < CPL; j++) {
+                const bool mj = jme == j;
+                if (__builtin_amdgcn_ballot_w64(mj) != 0) {
+                    const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo, acc[j], 0, 0, 0);
+                }
+            }
+        };
+        one(o.fl ? __builtin_ctz(o.fl) : 255, o.v0);
+        const uint32_t r1 = o.fl & (o.fl - 1u);
+        if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
+            one(r1 ? __builtin_ctz(r1) : 255, o.v1);
+            uint32_t rem = r1 & (r1 - 1u);
+            int slot = o.slot + 2;
+            while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
+                const bool has = rem != 0;
+                one(has ? __builtin_ctz(rem) : 255, has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4);
+                slot++;
+                rem &= rem - 1u;
+            }
+        }
+    };
+
+    // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.  A flagged chunk
+    // carries radius code 0 in the main plane, so its decoded value is exactly zero and only the verbatim
+    // value from the sideband contributes.
+    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const OutPre (&oc)[4]) {
         float4v sT[2];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
             decode_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, a);
             float4v s = zero4, so = zero4;
-            if (FLAGS) {
-                const uint32_t fw = h.kfl[u];
-                if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
-                    uint32_t fl;
-                    int slot;
-                    lane_flags(fw, h.ksb[u], fl, slot);
-#pragma unroll
-                    for (int j = 0; j < CPL; j++)
-                        if ((fl >> j) & 1u) a[j] = zero_h4;
-                    uint32_t rem = fl;
-                    while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
-                        const bool has = rem != 0;
-                        const int jme = has ? __builtin_ctz(rem) : 255;
-                        const half4 val = has ? outlier_chunk(p.Kc, DT, bh, slot) : zero_h4;
-                        slot++;
-                        rem &= rem - 1u;
-#pragma unroll
-                        for (int jj = 0; jj < CPL / 2; jj++) {
-                            const bool m0 = jme == 2 * jj, m1 = jme == 2 * jj + 1;
-                            if (__builtin_amdgcn_ballot_w64(m0 || m1) != 0)
-                                so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(m0 ? val : zero_h4, m1 ? val : zero_h4), qf[jj], so, 0, 0, 0);
-                        }
-                    }
-                }
-            }
 #pragma unroll
             for (int jj = 0; jj < CPL / 2; jj++)
                 s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
+            if (FLAGS) out_apply_k(oc[u], so);
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[e] * qmaxf : 0.f);
@@ -404,36 +467,8 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         // ---- O^T += V^T . P^T, both tiles in one MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
         half4 av[2][CPL];
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
+        for (int u = 0; u < 2; u++)
             decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, av[u]);
-            if (FLAGS) {
-                const uint32_t fw = h.vfl[u];
-                if (__builtin_amdgcn_ballot_w64(fw != 0) != 0) {
-                    uint32_t fl;
-                    int slot;
-                    lane_flags(fw, h.vsb[u], fl, slot);
-#pragma unroll
-                    for (int j = 0; j < CPL; j++)
-                        if ((fl >> j) & 1u) av[u][j] = zero_h4;
-                    uint32_t rem = fl;
-                    while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
-                        const bool has = rem != 0;
-                        const int jme = has ? __builtin_ctz(rem) : 255;
-                        const half4 val = has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4;
-                        slot++;
-                        rem &= rem - 1u;
-#pragma unroll
-                        for (int j = 0; j < CPL; j++) {
-                            const bool mj = jme == j;
-                            if (__builtin_amdgcn_ballot_w64(mj) != 0) {
-                                const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
-                                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo[u], acc[j], 0, 0, 0);
-                            }
-                        }
-                    }
-                }
-            }
-        }
         const half8 pp = cat8(pT[0], pT[1]);
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
@@ -441,15 +476,43 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
         }
+        if (FLAGS) {
+            out_apply_v(oc[2], pTo[0]);
+            out_apply_v(oc[3], pTo[1]);
+        }
     };
+
+    // sideband requests of one half-step: K tiles 0, 1, then V tiles 0, 1
+    auto issue_all = [&](const FlagTile &f, OutPre (&o)[4]) {
+        out_issue(p.Kc, f.kfl[0], f.ksb[0], o[0]);
+        out_issue(p.Kc, f.kfl[1], f.ksb[1], o[1]);
+        out_issue(p.Vc, f.vfl[0], f.vsb[0], o[2]);
+        out_issue(p.Vc, f.vfl[1], f.vsb[1], o[3]);
+    };
+    OutPre oc[4] = {};
+    if (FLAGS && t_begin < t_end) issue_all(f0, oc);
 
     for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
         FastTile<NW, AB, FLAGS, NH> nxt;
-        const bool more = t0 + STEP < t_end;
+        FlagTile f2 = {};
+        OutPre on[4] = {};
+        const bool more = t0 + STEP < t_end, more2 = t0 + 2 * STEP < t_end;
         if (more) load_super(t0 + STEP, nxt);
-        half_step(cur.h[0], t0);
-        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32);
-        if (more) cur = nxt;
+        if (FLAGS) {
+            // flags two steps ahead, sideband chunks one step ahead (their flags were requested a step ago)
+            if (more2) load_flags(t0 + 2 * STEP, f2);
+            if (more) issue_all(f1, on);
+        }
+        half_step(cur.h[0], t0, oc);
+        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, oc);
+        if (more) {
+            cur = nxt;
+            if (FLAGS) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) oc[i] = on[i];
+                f1 = f2;
+            }
+        }
     }
 
     // ---- merge the block's waves through LDS: rows of [d_h accumulators, m, l, pad] ----

@@ -314,7 +314,8 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
 
     // ---- packed rows ----
     if (a.main_plane || a.flag_plane || a.scale_plane) {
-        code_sh[tid] = (uint32_t)idx | ((uint32_t)rq << a.idx_bits);
+        // a flagged chunk is read from the sideband; its packed code keeps idx with radius code 0, which decodes to zero
+        code_sh[tid] = (uint32_t)idx | ((uint32_t)(flagged ? 0 : rq) << a.idx_bits);
         mask_sh[tid] = flagged ? 1u : 0u;
         __syncthreads();
         if (active) {

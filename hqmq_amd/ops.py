@@ -217,8 +217,9 @@ def dequant_packed(cache, T: Optional[int] = None, mode: int = 0) -> torch.Tenso
     return out
 
 
-def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int) -> int:
-    return int(L.lib().hqmq_attn_pick_splits(C.c_int(B), C.c_int(H_q), C.c_int(H_kv), C.c_int(T_q), C.c_int(T_kv)))
+def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int, ragged: bool = False) -> int:
+    return int(L.lib().hqmq_attn_pick_splits(C.c_int(B), C.c_int(H_q), C.c_int(H_kv), C.c_int(T_q), C.c_int(T_kv),
+                                             C.c_int(1 if ragged else 0)))
 
 
 def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None, causal: bool = False,
@@ -241,7 +242,7 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     if softmax_scale is None:
         softmax_scale = d_h ** -0.5
     if n_splits <= 0:
-        n_splits = pick_splits(B, Hq, Kc.H, Tq, max(T_kv, 1))
+        n_splits = pick_splits(B, Hq, Kc.H, Tq, max(T_kv, 1), kv_lens is not None)
     a = L.AttnArgs()
     a.Q, a.O = L.ptr(Q), L.ptr(O)
     a.q_sb, a.q_sh, a.q_st = Q.stride(0), Q.stride(1), Q.stride(2)

@@ -24,6 +24,8 @@
  *   sideband  = [B][H][sb_cap][4] in D: the flagged chunks verbatim, in
  *               (token, chunk) order; sb_tile_off[B][H][t_cap/16] = number of
  *               flagged chunks before token 16*i; sb_count[B][H] = total.
+ *               A flagged chunk's code keeps its idx but carries rq = 0, so that
+ *               it decodes to exactly zero and only the sideband value counts.
  *   s24_r3 -> 12+1 bits (48+4 B/token at d_h=128), s96_r4 -> 16+0 (64 B),
  *   s192_r6 -> 16+3 (64+12 B).
  */
@@ -181,7 +183,8 @@ typedef struct hqmq_attn_args {
     int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
-int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv);
+/* The n_splits hqmq_attn_fwd would choose; ragged = 1 when kv_len is passed (more, smaller blocks). */
+int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv, int ragged);
 int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream);
 /* Merge of the split-KV partials (m, l, acc) left in the workspace; hqmq_attn_fwd runs it unless skip_combine. */
 int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,

@@ -89,6 +89,12 @@ def test_flags_and_sideband_match_oracle(S, b_r, dn, d_h):
         want = CO.outlier_quantize(x, Jc, b_r, 3.0)
         assert int(want["mask"].sum()) > 0
         assert torch.equal(pt.flags[:, :, :T].cpu(), CO.pack_flags(want["mask"]))
+        # packed codes: a flagged chunk keeps its idx and carries radius code 0
+        rq0 = torch.where(want["mask"], torch.zeros_like(want["rq"]), want["rq"])
+        main, aux = CO.pack_rows(want["idx"], rq0, pt.idx_bits, pt.main_bits, pt.aux_bits)
+        assert torch.equal(pt.main[:, :, :T].cpu(), main)
+        if aux is not None:
+            assert torch.equal(pt.aux[:, :, :T].cpu(), aux)
         for b in range(B):
             for h in range(H):
                 sb, toff, cnt = CO.pack_sideband(x[b, h], want["mask"][b, h])
