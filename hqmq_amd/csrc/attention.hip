@@ -296,48 +296,47 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     }
 }
 
-// One block per output row (d_h <= 256 threads used): weights of the splits go to LDS first, then every thread
-// walks the partials of its element with independent loads.
+// One block per output row, one thread per element.  Every thread loads the (m, l, acc[e]) of up to 32 splits in
+// one batch of independent loads (the m and l of a split are the same addresses in all threads: broadcasts) and
+// merges them in registers, so the kernel costs one round trip to memory per 32 splits; no LDS, no barrier.
 __global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
                                                            int n_splits, int64_t osb, int64_t osh, int64_t ost) {
-    extern __shared__ float wsh[];          // [n_splits] weights
-    __shared__ float red_m[4], red_l[4];
     const int64_t row = blockIdx.x;
-    const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
-    const float *wp = ws + (size_t)row * n_splits * (d_h + 2);
-    float m = -INFINITY;
-    for (int s = threadIdx.x; s < n_splits; s += 256) {
-        const float v = wp[(size_t)s * (d_h + 2)];
-        wsh[s] = v;
-        m = fmaxf(m, v);
-    }
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if ((threadIdx.x & 63) == 0) red_m[threadIdx.x >> 6] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
-    float l = 0.f;
-    for (int s = threadIdx.x; s < n_splits; s += 256) {
-        const float f = m > -INFINITY ? exp2f(wsh[s] - m) : 0.f;
-        wsh[s] = f;
-        l = fmaf(wp[(size_t)s * (d_h + 2) + 1], f, l);
-    }
-    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
-    if ((threadIdx.x & 63) == 0) red_l[threadIdx.x >> 6] = l;
-    __syncthreads();
-    l = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
     const int e = threadIdx.x;
     if (e >= d_h) return;
-    const float *we = wp + 2 + e;
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int s = 0;
-    for (; s + 4 <= n_splits; s += 4) {
-        a0 = fmaf(we[(size_t)(s + 0) * (d_h + 2)], wsh[s + 0], a0);
-        a1 = fmaf(we[(size_t)(s + 1) * (d_h + 2)], wsh[s + 1], a1);
-        a2 = fmaf(we[(size_t)(s + 2) * (d_h + 2)], wsh[s + 2], a2);
-        a3 = fmaf(we[(size_t)(s + 3) * (d_h + 2)], wsh[s + 3], a3);
+    const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
+    const float *base = ws + (size_t)row * n_splits * (d_h + 2);
+    constexpr int SC = 32;
+    float M = -INFINITY, L = 0.f, A = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += SC) {
+        float ms[SC], ls[SC], as[SC];
+#pragma unroll
+        for (int i = 0; i < SC; i++) {
+            const bool ok = s0 + i < n_splits;
+            const float *q = base + (size_t)(ok ? s0 + i : s0) * (d_h + 2);
+            ms[i] = q[0];
+            ls[i] = q[1];
+            as[i] = q[2 + e];
+            if (!ok) { ms[i] = -INFINITY; ls[i] = 0.f; as[i] = 0.f; }
+        }
+        float mx = ms[0];
+#pragma unroll
+        for (int i = 1; i < SC; i++) mx = fmaxf(mx, ms[i]);
+        const float Mn = fmaxf(M, mx);
+        if (Mn > -INFINITY) {
+            const float f = exp2f(M - Mn);       // 0 while M is still -inf
+            L *= f;
+            A *= f;
+#pragma unroll
+            for (int i = 0; i < SC; i++) {
+                const float w = exp2f(ms[i] - Mn);
+                L = fmaf(ls[i], w, L);
+                A = fmaf(as[i], w, A);
+            }
+            M = Mn;
+        }
     }
-    for (; s < n_splits; s++) a0 = fmaf(we[(size_t)s * (d_h + 2)], wsh[s], a0);
-    store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, l > 0.f ? ((a0 + a1) + (a2 + a3)) / l : 0.f);
+    store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, L > 0.f ? A / L : 0.f);
 }
 
 static PackedDev to_dev(const hqmq_packed &k) {
@@ -400,7 +399,7 @@ extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int 
     if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(256), (size_t)n_splits * sizeof(float), (hipStream_t)stream,
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(d_h < 64 ? 64 : d_h), 0, (hipStream_t)stream,
                        (const float *)workspace, O,
                        dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
@@ -432,7 +431,7 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if (flags && (((uintptr_t)a->K.sideband % (4 * elt)) || ((uintptr_t)a->V.sideband % (4 * elt)))) return HQMQ_ERR_ALIGN;
 
     int n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv, a->kv_len != nullptr);
-    if (n_splits > 8192) return HQMQ_ERR_SHAPE;   // the merge keeps one weight per split in LDS
+    if (n_splits > 8192) return HQMQ_ERR_SHAPE;   // bound of hqmq_attn_combine
     if (n_splits > 1) {
         if (!a->workspace) return HQMQ_ERR_NULL;
         if (a->workspace_bytes < hqmq_attn_workspace_bytes(a->B, a->H_q, a->T_q, 4 * n, n_splits)) return HQMQ_ERR_WORKSPACE;
