@@ -72,6 +72,43 @@ __global__ void med_hist_kernel(const typename D::storage *x, int64_t xsb, int64
     }
 }
 
+// LEVEL 0 for large calls: the 32768 bins live in LDS (128 KB, one block per CU); a block adds only its non-zero
+// bins to the global histogram, a few thousand atomics instead of one per chunk.
+template <class D>
+__global__ __launch_bounds__(1024) void med_hist_lds_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int B,
+                                                            int H, int T, int n, uint32_t *ws) {
+    extern __shared__ uint32_t lh[];    // [kBins1] + 1 (NaN count)
+    const int h = blockIdx.y;
+    uint32_t *hist1 = ws + (size_t)h * kBins1;
+    uint32_t *state = ws + (size_t)H * kBins1 + (size_t)h * kState;
+    for (int i = threadIdx.x; i <= kBins1; i += 1024) lh[i] = 0;
+    __syncthreads();
+    const int64_t per_head = (int64_t)B * T * n;
+    for (int64_t g = (int64_t)blockIdx.x * 1024 + threadIdx.x; g < per_head; g += (int64_t)gridDim.x * 1024) {
+        int c, t, b;
+        if (per_head < 0x7fffffff) {
+            const uint32_t g32 = (uint32_t)g, bt = g32 / (uint32_t)n;
+            c = (int)(g32 - bt * (uint32_t)n);
+            b = (int)(bt / (uint32_t)T);
+            t = (int)(bt - (uint32_t)b * (uint32_t)T);
+        } else {
+            c = (int)(g % n);
+            const int64_t bt = g / n;
+            t = (int)(bt % T);
+            b = (int)(bt / T);
+        }
+        const float nrm = chunk_norm<D>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4);
+        if (is_nan(nrm)) atomicAdd(&lh[kBins1], 1u);
+        else atomicAdd(&lh[norm_bits<D>(nrm) >> 16], 1u);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < kBins1; i += 1024) {
+        const uint32_t v = lh[i];
+        if (v) atomicAdd(&hist1[i], v);
+    }
+    if (threadIdx.x == 0 && lh[kBins1]) atomicAdd(&state[0], lh[kBins1]);
+}
+
 // Finds the bins holding 0-based ranks r_lo <= r_hi in a histogram of `bins` counters.
 // One block of 1024 threads; results through shared memory.
 __device__ void select_two(const uint32_t *hist, int bins, int64_t r_lo, int64_t r_hi, uint32_t *key_lo, uint32_t *key_hi,
@@ -262,6 +299,79 @@ __global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage
     if (threadIdx.x == 0) sb_count[bh] = base_sh;
 }
 
+// ---- bulk appends (whole 16-row tiles from an aligned first row): three passes with one thread per tile / row ----
+// Pass 1: flagged chunks of every new tile -> sb_tile_off[tile] (a count for now).
+__global__ void tile_count_kernel(const uint8_t *flag_plane, int64_t t_cap, int row0, int T, int frb, int n_tiles, int32_t *sb_tile_off) {
+    const int bh = blockIdx.y;
+    const int64_t tiles = (t_cap + kTile - 1) / kTile;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_tiles) return;
+    const int r_begin = row0 + i * kTile, r_end = min(row0 + T, r_begin + kTile);
+    const uint8_t *fr = flag_plane + ((size_t)bh * t_cap + r_begin) * frb;
+    int cnt = 0;
+    for (int k = 0; k < (r_end - r_begin) * frb; k++) cnt += __popc((uint32_t)fr[k]);
+    sb_tile_off[(size_t)bh * tiles + (r_begin >> 4)] = cnt;
+}
+// Pass 2: one block per (b, h): counts -> sideband offsets (exclusive scan behind the chunks already stored).
+__global__ __launch_bounds__(1024) void tile_scan_kernel(int64_t t_cap, int row0, int n_tiles, int32_t *sb_tile_off, int32_t *sb_count) {
+    __shared__ int part[1024];
+    const int bh = blockIdx.x;
+    const int64_t tiles = (t_cap + kTile - 1) / kTile;
+    int32_t *to = sb_tile_off + (size_t)bh * tiles + (row0 >> 4);
+    const int per = (n_tiles + 1023) / 1024;
+    const int i0 = threadIdx.x * per, i1 = min(n_tiles, i0 + per);
+    int s = 0;
+    for (int i = i0; i < i1; i++) s += to[i];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int v = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    const int base = sb_count[bh];
+    int run = base + part[threadIdx.x] - s;
+    for (int i = i0; i < i1; i++) {
+        const int c = to[i];
+        to[i] = run;
+        run += c;
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) sb_count[bh] = base + part[1023];
+}
+// Pass 3: one thread per new row copies the row's flagged chunks behind those of the tile's earlier rows.
+template <class D>
+__global__ void tile_copy_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H, int T, int n,
+                                 const uint8_t *flag_plane, int64_t t_cap, int row0, typename D::storage *sideband, int64_t sb_cap,
+                                 const int32_t *sb_tile_off, int32_t *overflow) {
+    using ST = typename D::storage;
+    const int bh = blockIdx.y, b = bh / H, h = bh - b * H;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    const int frb = (n + 7) >> 3;
+    const int64_t tiles = (t_cap + kTile - 1) / kTile;
+    const int row = row0 + t, tile_row = row & ~(kTile - 1);
+    const uint8_t *fr = flag_plane + ((size_t)bh * t_cap + row) * frb;
+    int own = 0;
+    for (int k = 0; k < frb; k++) own += __popc((uint32_t)fr[k]);
+    if (!own) return;
+    int before = sb_tile_off[(size_t)bh * tiles + (row >> 4)];
+    const uint8_t *f0 = flag_plane + ((size_t)bh * t_cap + tile_row) * frb;
+    for (int k = 0; k < (row - tile_row) * frb; k++) before += __popc((uint32_t)f0[k]);
+    const ST *xr = x + b * xsb + h * xsh + (int64_t)t * xst;
+    int k = before;
+    for (int c = 0; c < n; c++) {
+        if ((fr[c >> 3] >> (c & 7)) & 1) {
+            if (k < sb_cap) {
+                ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
+                for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
+            } else *overflow = 1;
+            k++;
+        }
+    }
+}
+
 }  // namespace hqmq
 
 using namespace hqmq;
@@ -281,7 +391,16 @@ static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B
     const int64_t per_head = (int64_t)B * T * n;
     int gx = (int)((per_head + 255) / 256);
     if (gx > 2048) gx = 2048;
-    hipLaunchKernelGGL((med_hist_kernel<D, 0>), dim3(gx, H), dim3(256), 0, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
+    if (per_head >= (1 << 18)) {
+        const size_t lds = (size_t)(kBins1 + 1) * sizeof(uint32_t);
+        hipError_t e = hipFuncSetAttribute((const void *)med_hist_lds_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        int gl = (int)((per_head + 16383) / 16384);
+        if (gl > 128) gl = 128;
+        hipLaunchKernelGGL(med_hist_lds_kernel<D>, dim3(gl, H), dim3(1024), lds, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
+    } else {
+        hipLaunchKernelGGL((med_hist_kernel<D, 0>), dim3(gx, H), dim3(256), 0, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
+    }
     hipLaunchKernelGGL(med_select1_kernel<D>, dim3(H), dim3(1024), 0, st, ws, H, per_head, mult, median, (ST *)thr, n_out);
     if (f32) {
         hipLaunchKernelGGL((med_hist_kernel<D, 1>), dim3(gx, H), dim3(256), 0, st, (const ST *)x, xsb, xsh, xst, B, H, T, n, ws);
@@ -320,6 +439,24 @@ extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x
     if (B < 1 || H < 1 || T < 0 || n_chunks < 1 || t_cap < 1 || sb_cap < 1 || t_off < 0) return HQMQ_ERR_SHAPE;
     if (T == 0) return HQMQ_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (!pos && (t_off % kTile) == 0 && T >= 512 && (int64_t)t_off + T <= t_cap && B * H <= 65535) {
+        const int n_tiles = (T + kTile - 1) / kTile, frb = (n_chunks + 7) >> 3;
+        hipLaunchKernelGGL(tile_count_kernel, dim3((n_tiles + 255) / 256, B * H), dim3(256), 0, st, flag_plane, t_cap, t_off, T, frb,
+                           n_tiles, sb_tile_off);
+        hipLaunchKernelGGL(tile_scan_kernel, dim3(B * H), dim3(1024), 0, st, t_cap, t_off, n_tiles, sb_tile_off, sb_count);
+        dim3 cgrid((T + 255) / 256, B * H);
+#define COPY(DT, ST)                                                                                                          \
+    hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T,    \
+                       n_chunks, flag_plane, t_cap, t_off, (ST *)sideband, sb_cap, sb_tile_off, overflow)
+        switch (dtype) {
+            case HQMQ_F32: COPY(F32, float); break;
+            case HQMQ_F16: COPY(F16, uint16_t); break;
+            case HQMQ_BF16: COPY(BF16, uint16_t); break;
+            default: return HQMQ_ERR_DTYPE;
+        }
+#undef COPY
+        return hip_status(hipGetLastError());
+    }
     dim3 grid(B * H), block(1024);
 #define LAUNCH(DT, ST)                                                                                                      \
     hipLaunchKernelGGL(compact_kernel<DT>, grid, block, 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T, n_chunks, \

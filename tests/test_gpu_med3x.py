@@ -12,7 +12,7 @@ DEV = "cuda"
 
 
 @pytest.mark.parametrize("dn", ["fp32", "fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(2, 3, 70, 64), (1, 2, 5, 12), (1, 1, 1, 128), (3, 4, 257, 128)])
+@pytest.mark.parametrize("shape", [(2, 3, 70, 64), (1, 2, 5, 12), (1, 1, 1, 128), (3, 4, 257, 128), (2, 2, 4200, 128)])
 def test_median_threshold_count(dn, shape):
     """Even and odd chunk counts, tiny calls (one decode token), all dtypes (fp32 takes the two-pass select)."""
     from hqmq_amd import ops
@@ -107,6 +107,30 @@ def test_flags_and_sideband_match_oracle(S, b_r, dn, d_h):
         assert bit_equal(ops.dequant_packed(pt, T, mode=0), dense)
     assert cache.nbytes() == sum(pt.B * pt.H * T * pt.row_bytes() + int(pt.sb_count.sum()) * 4 * pt.scale.element_size()
                                  for pt in (cache.K, cache.V))
+
+
+@pytest.mark.parametrize("dn,d_h", [("fp16", 128), ("bf16", 64)])
+def test_bulk_append_compaction_then_more_appends(dn, d_h):
+    """A long first append takes the tile-parallel compaction (ragged last tile), the following appends the
+    in-order one; flags, sideband order, tile offsets and counts equal the oracle's over all rows."""
+    import hqmq
+    dt = DT[dn]
+    B, H, T1, T2, T3 = 2, 3, 1000, 24, 1
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=24, radius_bits=3, device=DEV))
+    cache = w.new_cache(B, T1 + T2 + T3, d_h, dt, 0, sideband_frac=0.5)
+    ks = kv_input((B, H, T1 + T2 + T3, d_h), dt, seed=17, outlier_p=0.04)
+    cuts = [0, T1, T1 + T2, T1 + T2 + T3]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        w.append(cache, ks[:, :, a:b].to(DEV), ks[:, :, a:b].to(DEV), 0)
+    cache.K.check_overflow()
+    masks = torch.cat([CO.med3x(ks[:, :, a:b].contiguous())["mask"] for a, b in zip(cuts[:-1], cuts[1:])], dim=2)
+    assert torch.equal(cache.K.flags[:, :, :cuts[-1]].cpu(), CO.pack_flags(masks))
+    for b in range(B):
+        for h in range(H):
+            sb, toff, cnt = CO.pack_sideband(ks[b, h], masks[b, h])
+            assert int(cache.K.sb_count[b, h]) == cnt and cnt > 0
+            assert bit_equal(cache.K.sideband[b, h, :cnt], sb)
+            assert torch.equal(cache.K.sb_tile_off[b, h, :toff.numel()].cpu(), toff)
 
 
 def test_decode_appends_keep_sideband_consistent():
