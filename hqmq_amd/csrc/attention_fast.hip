@@ -11,7 +11,8 @@
 //   O^T += V^T . P^T  v_mfma_f32_16x16x32_f16 over two tiles (32 tokens) at a time.
 // Row j of the V-side product is d = (grp * CPL + j) * 4 + e, the order the epilogue writes back.
 // Scores are kept as S^T * rs; 1/qmax is folded into the softmax scale and the epilogue.  Outlier chunks
-// (flag bit set) are zeroed in the decoded operand and enter through extra MFMAs with their verbatim values.
+// (flag bit set) carry radius code 0, so they decode to zero, and enter through extra MFMAs with their
+// verbatim sideband values.
 #include "attention_common.h"
 
 namespace hqmq {
