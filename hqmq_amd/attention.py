@@ -94,16 +94,19 @@ def fused_attention(
 
 def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = False, softmax_scale: Optional[float] = None,
                            kv_lens: Optional[torch.Tensor] = None, causal_offset: int = 0, n_splits: int = 0,
-                           T_kv: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           T_kv: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                           force_generic: bool = False) -> torch.Tensor:
     """Fused attention straight from the bit-packed cache (the fast path).
 
     Decode: T_q = 1, causal=False.  Chunked prefill: causal=True with causal_offset = number of
     cached tokens before the chunk (bottom-right alignment).  Ragged batches pass kv_lens (int32 [B]).
+    force_generic runs the layout-generic kernel where a specialised one exists (a second implementation
+    of the same arithmetic, used by the tests).
     """
     if T_kv is None:
         T_kv = cache.K.t_cap if kv_lens is not None else cache.K.length
     return ops.attn_fwd(Q, cache.K, cache.V, T_kv, kv_lens=kv_lens, causal=causal, causal_offset=causal_offset,
-                        softmax_scale=softmax_scale, n_splits=n_splits, out=out)
+                        softmax_scale=softmax_scale, n_splits=n_splits, out=out, force_generic=force_generic)
 
 
 def fused_attention_reference(

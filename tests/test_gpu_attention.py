@@ -236,3 +236,38 @@ def test_argument_checks():
         hqmq.fused_attention_packed(torch.randn(1, 4, 1, 64, device=DEV), cache)              # dtype mismatch
     with pytest.raises(hqmq.HqmqError):
         q.append(cache, x, x, 0)                                                              # capacity exceeded
+
+
+@pytest.mark.parametrize("cfg", [3, 5])
+def test_config3_and_5_full_size_properties(cfg):
+    """BASELINE configs 3 (28/4 heads, batch 8, 32k, s192_r6 + Med3x, fp16, 2 % of K chunks x50-200) and
+    5 (64/8 heads, d_h 64, batch 4, 131072, s96_r4 + Med3x, bf16, 1 % of chunks x100) at full size: agreement with
+    dense fp32 attention over the dequantized cache, split invariance, and the specialised kernel against the
+    layout-generic one.  Outputs reach |O| ~ 4 (config 3) and ~ 350 (config 5), so bounds are relative to that."""
+    import hqmq
+    from hqmq_amd.bench_configs import dense_check, synth
+    if cfg == 3:
+        B, Hq, Hkv, d, S, b_r, dt, T = 8, 28, 4, 128, 192, 6, torch.float16, 32768
+        k, v = synth((B, Hkv, T, d), dt, 31, outlier_p=0.02), synth((B, Hkv, T, d), dt, 32)
+    else:
+        B, Hq, Hkv, d, S, b_r, dt, T = 4, 64, 8, 64, 96, 4, torch.bfloat16, 131072
+        k = synth((B, Hkv, T, d), dt, 51, outlier_p=0.01, gain=(100.0, 100.0))
+        v = synth((B, Hkv, T, d), dt, 52, outlier_p=0.01, gain=(100.0, 100.0))
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV), C=3.0)
+    cache = w.new_cache(B, T, d, dt, 0, sideband_frac=0.125)
+    w.append(cache, k, v, 0)
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    del k, v
+    rate = float(cache.K.sb_count.sum()) / (B * Hkv * T * d / 4)
+    assert 0.005 < rate < 0.03
+    Q = torch.randn(B, Hq, 1, d, generator=torch.Generator().manual_seed(7)).to(dt).to(DEV)
+    err, ref_max = dense_check(Q, cache, None, T)
+    scale = max(1.0, ref_max)
+    assert err < 2e-3 * scale, (err, ref_max)
+    O = hqmq.fused_attention_packed(Q, cache)
+    for ns in (1, 5):
+        o = hqmq.fused_attention_packed(Q, cache, n_splits=ns)
+        assert (o.float() - O.float()).abs().max().item() < 1e-3 * scale
+    og = hqmq.fused_attention_packed(Q, cache, force_generic=True)
+    assert (og.float() - O.float()).abs().max().item() < 1e-3 * scale
