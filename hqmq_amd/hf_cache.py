@@ -1,0 +1,140 @@
+"""Hugging Face `transformers` caches over the HQMQ path.
+
+QuantizedCache
+    The reference's cache hook (src/model_utils.py:22-32 of the reference): every K, V that is appended goes
+    through `quantize_K` / `quantize_V` (fake quantization on the GPU kernels) into an ordinary DynamicCache.
+
+PackedQuantizedCache  +  attn_implementation="hqmq_packed"
+    What the reference describes but does not have: each layer keeps the bit-packed planes (`PackedKV`), an
+    append quantizes the new tokens straight into them, and attention reads the compressed cache with the fused
+    kernel.  `update` returns only the new tokens' K, V (nothing dense is kept); the tensors it returns carry a
+    reference to their layer, which is how the attention function finds the planes.
+
+    model.set_attn_implementation("hqmq_packed")
+    cache = PackedQuantizedCache(quantizer, max_tokens=4096)
+    out = model(input_ids, past_key_values=cache, use_cache=True)
+
+Limits: unpadded batches (every sequence of the batch has the same length; the causal mask is the only mask),
+no cache cropping / beam reordering.  This module imports `transformers`; nothing else in the package does.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from transformers import AttentionInterface, DynamicCache
+from transformers.cache_utils import DynamicLayer
+
+from ._lib import HqmqError
+from .attention import fused_attention_packed
+from .quantizer import KVQuantizer
+
+ATTN_NAME = "hqmq_packed"
+
+
+class QuantizedCache(DynamicCache):
+    """DynamicCache that fake-quantizes K, V on every update (same class as the reference's)."""
+
+    def __init__(self, quantizer: KVQuantizer):
+        super().__init__()
+        self.quantizer = quantizer
+
+    def update(self, key_states, value_states, layer_idx, *args, **kwargs):
+        k_q = self.quantizer.quantize_K(key_states, layer_idx)
+        v_q = self.quantizer.quantize_V(value_states, layer_idx)
+        return super().update(k_q, v_q, layer_idx, *args, **kwargs)
+
+
+class PackedLayer(DynamicLayer):
+    """One layer's compressed K and V."""
+
+    def __init__(self, quantizer, layer_idx: int, max_tokens: int, sideband_frac: float):
+        super().__init__()
+        self.quantizer, self.layer_idx, self.max_tokens, self.sideband_frac = quantizer, layer_idx, max_tokens, sideband_frac
+        self.packed = None
+        self.n_tokens = 0
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, *args, **kwargs):
+        if self.packed is None:
+            B, _, _, d_h = key_states.shape
+            kw = {"sideband_frac": self.sideband_frac} if hasattr(self.quantizer, "median_mult") else {}
+            self.packed = self.quantizer.new_cache(B, self.max_tokens, d_h, key_states.dtype, self.layer_idx, **kw)
+            self.dtype, self.device = key_states.dtype, key_states.device
+            self.keys = self.values = torch.empty(0, dtype=self.dtype, device=self.device)
+            self.is_initialized = True
+        if self.n_tokens + key_states.shape[2] > self.packed.K.t_cap:
+            raise HqmqError(f"PackedQuantizedCache holds {self.packed.K.t_cap} tokens per sequence; raise max_tokens")
+        self.quantizer.append(self.packed, key_states, value_states, self.layer_idx)
+        self.n_tokens += key_states.shape[2]
+        key_states.hqmq_layer = self          # how hqmq_packed_attention finds the planes
+        return key_states, value_states
+
+    def get_seq_length(self) -> int:
+        return self.n_tokens
+
+    def get_max_length(self) -> int:
+        return self.max_tokens
+
+    def crop(self, *args, **kwargs):
+        raise NotImplementedError("a packed cache cannot be cropped")
+
+    def batch_repeat_interleave(self, repeats: int) -> None:
+        raise NotImplementedError("a packed cache cannot be repeated along the batch")
+
+    def batch_select_indices(self, indices: torch.Tensor) -> None:
+        raise NotImplementedError("a packed cache cannot be re-indexed along the batch")
+
+
+class PackedQuantizedCache(DynamicCache):
+    """Keeps every layer bit-packed; use with attn_implementation="hqmq_packed"."""
+
+    def __init__(self, quantizer, max_tokens: int, sideband_frac: float = 0.125):
+        super().__init__()
+        if not hasattr(quantizer, "append") or not hasattr(quantizer, "new_cache"):
+            raise TypeError("PackedQuantizedCache needs an HQMQ quantizer (HQMQ(...) or with_outlier_extraction(HQMQ(...)))")
+        self.quantizer, self.max_tokens, self.sideband_frac = quantizer, int(max_tokens), sideband_frac
+
+    def update(self, key_states, value_states, layer_idx, *args, **kwargs):
+        while len(self.layers) <= layer_idx:
+            self.layers.append(PackedLayer(self.quantizer, len(self.layers), self.max_tokens, self.sideband_frac))
+        return self.layers[layer_idx].update(key_states, value_states, *args, **kwargs)
+
+    def check_overflow(self) -> None:
+        """Raises if any layer ran out of outlier sideband room (one device read per tensor): allocate with a
+        larger sideband_frac for data with many flagged chunks."""
+        for layer in self.layers:
+            if layer.packed is not None:
+                layer.packed.K.check_overflow()
+                layer.packed.V.check_overflow()
+
+    def nbytes(self) -> int:
+        """Compressed bytes held (all layers, rows written so far)."""
+        return sum(layer.packed.nbytes(layer.n_tokens) for layer in self.layers if layer.packed is not None)
+
+
+def hqmq_packed_attention(module, query, key, value, attention_mask, dropout: float = 0.0,
+                          scaling: Optional[float] = None, **kwargs):
+    """attention_interface function: causal attention of `query` over the packed cache of `key`'s layer."""
+    layer = getattr(key, "hqmq_layer", None)
+    if layer is None:
+        raise HqmqError('attn_implementation="hqmq_packed" needs past_key_values=PackedQuantizedCache(...)')
+    if dropout:
+        raise NotImplementedError("attention dropout is not supported on the packed path")
+    t_q = query.shape[2]
+    out = fused_attention_packed(query, layer.packed, causal=True, causal_offset=layer.n_tokens - t_q,
+                                 softmax_scale=scaling, T_kv=layer.n_tokens)
+    return out.transpose(1, 2).contiguous(), None
+
+
+def register() -> str:
+    """Registers the attention function (and the mask builder it shares with sdpa) under ATTN_NAME."""
+    AttentionInterface.register(ATTN_NAME, hqmq_packed_attention)
+    try:
+        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+        AttentionMaskInterface.register(ATTN_NAME, sdpa_mask)
+    except ImportError:          # older transformers build the mask without a per-implementation table
+        pass
+    return ATTN_NAME
+
+
+register()

@@ -1,0 +1,66 @@
+"""The HF cache hook on a small random Llama: the packed cache + fused attention against the reference-style
+fake-quantizing cache + dense attention, prefill and decode steps, with and without Med3x."""
+import pytest
+import torch
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
+DEV = "cuda"
+
+
+def tiny_llama(dtype):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg = LlamaConfig(vocab_size=256, hidden_size=512, intermediate_size=1024, num_hidden_layers=3, num_attention_heads=8,
+                      num_key_value_heads=2, head_dim=64, max_position_embeddings=1024)
+    torch.manual_seed(0)
+    return LlamaForCausalLM(cfg).to(dtype).to(DEV).eval()
+
+
+@pytest.mark.parametrize("med3x", [False, True])
+@pytest.mark.parametrize("dn", ["fp16", "bf16"])
+def test_packed_cache_matches_fake_quant_cache(dn, med3x):
+    import hqmq
+    from transformers import DynamicCache
+    from src.model_utils import ATTN_NAME, PackedQuantizedCache, QuantizedCache
+    dt = {"fp16": torch.float16, "bf16": torch.bfloat16}[dn]
+    model = tiny_llama(dt)
+    q = hqmq.HQMQ(n_layers=3, n_heads=2, secondary_size=96, radius_bits=4, device=DEV)
+    if med3x:
+        q = hqmq.with_outlier_extraction(q, C=3.0)
+        with torch.no_grad():                      # outlier channels: two chunks of K and one of V per KV head
+            for layer in model.model.layers:
+                layer.self_attn.k_proj.weight[8:16] *= 12.0
+                layer.self_attn.k_proj.weight[64 + 20:64 + 24] *= 12.0
+                layer.self_attn.v_proj.weight[40:44] *= 12.0
+    ids = torch.randint(0, 256, (2, 150), generator=torch.Generator().manual_seed(1)).to(DEV)
+    steps = 6
+
+    def run(cache):
+        logits = []
+        with torch.no_grad():
+            out = model(ids[:, :-steps], past_key_values=cache, use_cache=True)
+            logits.append(out.logits[:, -1].float())
+            for s in range(steps):
+                out = model(ids[:, -steps + s:ids.shape[1] - steps + s + 1], past_key_values=cache, use_cache=True)
+                logits.append(out.logits[:, -1].float())
+        return torch.stack(logits)
+
+    model.set_attn_implementation("sdpa")
+    want = run(QuantizedCache(q))                      # reference behaviour: fake-quantized dense cache
+    plain = run(DynamicCache())                        # unquantized, to size the effect of quantization
+    model.set_attn_implementation(ATTN_NAME)
+    packed = PackedQuantizedCache(q, max_tokens=256, sideband_frac=0.5)    # the planted channels flag ~20 % of K chunks
+    got = run(packed)
+    packed.check_overflow()
+    assert packed.get_seq_length() == ids.shape[1]
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    quant_effect = (want - plain).abs().max().item()
+    # the two paths hold the same codes; they differ by the decode rounding convention (<= 1 ulp of the cache
+    # dtype) and by fp16-vs-cache-dtype products inside attention, far less than quantization itself moves the logits
+    print(f"{dn} med3x={med3x}: max|logit| {scale:.3f}, packed vs fake-quant {err:.2e}, quantized vs unquantized {quant_effect:.2e}")
+    assert err < (0.02 if dn == "fp16" else 0.06) * scale and err < 0.5 * quant_effect, (err, scale, quant_effect)
+    if med3x:
+        assert all(int(layer.packed.K.sb_count.sum()) > 0 and int(layer.packed.V.sb_count.sum()) > 0 for layer in packed.layers)
+    # compressed size: 4 bits/value of codes + the per-token scale (+ flags and sideband with Med3x)
+    dense_bytes = 3 * 2 * 2 * 2 * ids.shape[1] * 64 * 2
+    assert packed.nbytes() < (0.6 if med3x else 0.36) * dense_bytes
