@@ -42,7 +42,7 @@ class Packed(C.Structure):
     _fields_ = [
         ("main_plane", vp), ("aux_plane", vp), ("flag_plane", vp), ("scale_plane", vp),
         ("scale_sb", i64), ("scale_sh", i64), ("scale_st", i64),
-        ("sideband", vp), ("sb_tile_off", vp), ("sb_cap", i64),
+        ("sideband", vp), ("sb_tile_off", vp), ("sb_cap", i64), ("sb_coord", vp), ("sb_count", vp),
         ("joint", vp), ("joint_sh", i64), ("K", C.c_int),
     ]
 

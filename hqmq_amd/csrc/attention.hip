@@ -341,7 +341,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void
 
 static PackedDev to_dev(const hqmq_packed &k) {
     return PackedDev{k.main_plane, k.aux_plane, k.flag_plane, k.scale_plane, k.scale_sb, k.scale_sh, k.scale_st,
-                     k.sideband, k.sb_tile_off, k.sb_cap, k.joint, k.joint_sh, k.K};
+                     k.sideband, k.sb_tile_off, k.sb_cap, k.sb_coord, k.sb_count, k.joint, k.joint_sh, k.K};
 }
 
 template <int CPL, int MB>

@@ -17,6 +17,8 @@ struct PackedDev {
     const void *sideband;
     const int32_t *sb_tile_off;
     int64_t sb_cap;
+    const uint16_t *sb_coord;
+    const int32_t *sb_count;
     const void *joint;
     int64_t jsh;
     int K;

@@ -250,7 +250,7 @@ template <class D>
 __global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H,
                                                         int T, int n, const uint8_t *flag_plane, int64_t t_cap, int t_off,
                                                         const int32_t *pos, typename D::storage *sideband, int64_t sb_cap,
-                                                        int32_t *sb_tile_off, int32_t *sb_count, int32_t *overflow) {
+                                                        int32_t *sb_tile_off, int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord) {
     using ST = typename D::storage;
     __shared__ int scan[1024];
     __shared__ int base_sh;
@@ -287,6 +287,7 @@ __global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage
                     if (k < sb_cap) {
                         ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                         for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
+                        if (sb_coord) sb_coord[(size_t)bh * sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
                     } else *overflow = 1;
                     k++;
                 }
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(int64_t t_cap, int row0
 template <class D>
 __global__ void tile_copy_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H, int T, int n,
                                  const uint8_t *flag_plane, int64_t t_cap, int row0, typename D::storage *sideband, int64_t sb_cap,
-                                 const int32_t *sb_tile_off, int32_t *overflow) {
+                                 const int32_t *sb_tile_off, int32_t *overflow, uint16_t *sb_coord) {
     using ST = typename D::storage;
     const int bh = blockIdx.y, b = bh / H, h = bh - b * H;
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -366,6 +367,7 @@ __global__ void tile_copy_kernel(const typename D::storage *x, int64_t xsb, int6
             if (k < sb_cap) {
                 ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                 for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
+                if (sb_coord) sb_coord[(size_t)bh * sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
             } else *overflow = 1;
             k++;
         }
@@ -434,7 +436,7 @@ extern "C" int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x
 extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
                                     int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
                                     const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off,
-                                    int32_t *sb_count, int32_t *overflow, void *stream) {
+                                    int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord, void *stream) {
     if (!x || !flag_plane || !sideband || !sb_tile_off || !sb_count || !overflow) return HQMQ_ERR_NULL;
     if (B < 1 || H < 1 || T < 0 || n_chunks < 1 || t_cap < 1 || sb_cap < 1 || t_off < 0) return HQMQ_ERR_SHAPE;
     if (T == 0) return HQMQ_OK;
@@ -447,7 +449,7 @@ extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x
         dim3 cgrid((T + 255) / 256, B * H);
 #define COPY(DT, ST)                                                                                                          \
     hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T,    \
-                       n_chunks, flag_plane, t_cap, t_off, (ST *)sideband, sb_cap, sb_tile_off, overflow)
+                       n_chunks, flag_plane, t_cap, t_off, (ST *)sideband, sb_cap, sb_tile_off, overflow, sb_coord)
         switch (dtype) {
             case HQMQ_F32: COPY(F32, float); break;
             case HQMQ_F16: COPY(F16, uint16_t); break;
@@ -460,7 +462,7 @@ extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x
     dim3 grid(B * H), block(1024);
 #define LAUNCH(DT, ST)                                                                                                      \
     hipLaunchKernelGGL(compact_kernel<DT>, grid, block, 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T, n_chunks, \
-                       flag_plane, t_cap, t_off, pos, (ST *)sideband, sb_cap, sb_tile_off, sb_count, overflow)
+                       flag_plane, t_cap, t_off, pos, (ST *)sideband, sb_cap, sb_tile_off, sb_count, overflow, sb_coord)
     switch (dtype) {
         case HQMQ_F32: LAUNCH(F32, float); break;
         case HQMQ_F16: LAUNCH(F16, uint16_t); break;

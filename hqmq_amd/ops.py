@@ -163,7 +163,7 @@ def outlier_compact(x: torch.Tensor, cache, t_off: int = 0, pos: Optional[torch.
             L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
             C.c_int(T), C.c_int(d_h // 4), L.ptr(cache.flags), L.i64(cache.t_cap), C.c_int(t_off), L.ptr(pos),
             L.ptr(cache.sideband), L.i64(cache.sb_cap), L.ptr(cache.sb_tile_off), L.ptr(cache.sb_count),
-            L.ptr(cache.sb_overflow), L.stream_ptr(dev)), "hqmq_outlier_compact")
+            L.ptr(cache.sb_overflow), L.ptr(cache.sb_coord), L.stream_ptr(dev)), "hqmq_outlier_compact")
 
 
 def _i32(t: torch.Tensor) -> torch.Tensor:

@@ -45,13 +45,15 @@ class PackedTensor:
         self.joint = joint
         self.length = 0                      # rows written when all sequences advance together
         self.lengths: Optional[torch.Tensor] = None  # per-sequence rows (int32, device) for ragged batches
-        self.flags = self.sideband = self.sb_tile_off = self.sb_count = self.sb_overflow = None
+        self.flags = self.sideband = self.sb_tile_off = self.sb_count = self.sb_overflow = self.sb_coord = None
         self.sb_cap = 0
         if outliers:
             self.flags = torch.zeros(B, H, self.t_cap, (n + 7) // 8, **z)
             self.sb_cap = max(64, int(self.t_cap * n * sideband_frac))
             self.sideband = torch.zeros(B, H, self.sb_cap, 4, dtype=dtype, device=self.device)
-            self.sb_tile_off = torch.zeros(B, H, self.t_cap // TILE, dtype=torch.int32, device=self.device)
+            # tiles not yet written read as "no entries"
+            self.sb_tile_off = torch.full((B, H, self.t_cap // TILE), 0x7fffffff, dtype=torch.int32, device=self.device)
+            self.sb_coord = torch.zeros(B, H, self.sb_cap, dtype=torch.int16, device=self.device)
             self.sb_count = torch.zeros(B, H, dtype=torch.int32, device=self.device)
             self.sb_overflow = torch.zeros(1, dtype=torch.int32, device=self.device)
 
@@ -82,6 +84,7 @@ class PackedTensor:
         s.scale_plane = L.ptr(self.scale)
         s.scale_sb, s.scale_sh, s.scale_st = self.scale.stride(0), self.scale.stride(1), self.scale.stride(2)
         s.sideband, s.sb_tile_off, s.sb_cap = L.ptr(self.sideband), L.ptr(self.sb_tile_off), self.sb_cap
+        s.sb_coord, s.sb_count = L.ptr(self.sb_coord), L.ptr(self.sb_count)
         s.joint, s.joint_sh, s.K = L.ptr(self.joint), self.joint.stride(0), self.joint.shape[1]
         return s
 

@@ -23,7 +23,8 @@
  *   flags row = 1 bit per chunk (Med3x outlier), n/8 bytes            (optional)
  *   sideband  = [B][H][sb_cap][4] in D: the flagged chunks verbatim, in
  *               (token, chunk) order; sb_tile_off[B][H][t_cap/16] = number of
- *               flagged chunks before token 16*i; sb_count[B][H] = total.
+ *               flagged chunks before token 16*i (INT32_MAX for tiles not yet written);
+ *               sb_count[B][H] = total; sb_coord[B][H][sb_cap] = (token & 15) << 8 | chunk per entry.
  *               A flagged chunk's code keeps its idx but carries rq = 0, so that
  *               it decodes to exactly zero and only the sideband value counts.
  *   s24_r3 -> 12+1 bits (48+4 B/token at d_h=128), s96_r4 -> 16+0 (64 B),
@@ -115,11 +116,14 @@ int hqmq_outlier_mask(const void *x, int64_t x_stride_b, int64_t x_stride_h, int
 
 /* Compact the flagged chunks of rows [row0, row0+T) into the sideband.
  * No counterpart in the reference (its wrapper keeps a dense tensor).
- * Rows must be appended in order; row0 = (pos ? pos[b] : 0) + t_off. */
+ * Rows must be appended in order; row0 = (pos ? pos[b] : 0) + t_off.
+ * sb_coord [B][H][sb_cap] (may be NULL): (row & 15) << 8 | chunk of every sideband entry, which lets the
+ * specialised attention kernels walk the sideband densely; sb_tile_off must start out as INT32_MAX (tiles not
+ * yet written read as "no entries"). */
 int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype,
                          int B, int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
                          const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off, int32_t *sb_count,
-                         int32_t *overflow, void *stream);
+                         int32_t *overflow, uint16_t *sb_coord, void *stream);
 
 /* Dense decode of unpacked codes: out = joint[h, idx] * ((rq * rs) / qmax) in D.
  * Replaces hqmq_decode_triton (src/quantizers/hqmq_kernel.py:102-132) with the
@@ -146,6 +150,8 @@ typedef struct hqmq_packed {
     const void *sideband;     /* NULL when flag_plane is NULL */
     const int32_t *sb_tile_off;
     int64_t sb_cap;
+    const uint16_t *sb_coord; /* [B][H][sb_cap] entry coordinates, or NULL (then the layout-generic kernel is used) */
+    const int32_t *sb_count;  /* [B][H] entries in use */
     const void *joint;        /* [H][K][4] D */
     int64_t joint_sh;         /* element stride between heads */
     int K;                    /* codewords in joint */

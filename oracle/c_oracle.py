@@ -158,6 +158,16 @@ def pack_flags(mask: torch.Tensor) -> torch.Tensor:
     return flags.view(*lead, st)
 
 
+def pack_coords(mask_bh: torch.Tensor) -> torch.Tensor:
+    """One (b, h) stream: mask (T, n) -> int16 coordinates (t & 15) << 8 | c of the sideband entries."""
+    T, n = mask_bh.shape
+    m8 = mask_bh.to(torch.uint8).contiguous()
+    out = torch.zeros(max(int(m8.sum()), 1), dtype=torch.int16)
+    lib().orc_pack_coords.restype = C.c_long
+    cnt = lib().orc_pack_coords(_p(m8), C.c_long(T), C.c_int(n), _p(out))
+    return out[:cnt]
+
+
 def pack_sideband(x_bh: torch.Tensor, mask_bh: torch.Tensor):
     """One (b, h) stream: x (T, 4n), mask (T, n) -> (sideband (count, 4), tile_off (ceil(T/16),), count)."""
     T, n = mask_bh.shape

@@ -353,6 +353,15 @@ void orc_pack_flags(const uint8_t *mask, long rows, int n, uint8_t *flags, long 
             if (mask[r * n + c]) flags[r * stride + (c >> 3)] |= (uint8_t)(1u << (c & 7));
     }
 }
+/* Coordinates of the sideband entries of one (b, h) stream, in the same order: (t & 15) << 8 | c. */
+long orc_pack_coords(const uint8_t *mask, long T, int n, uint16_t *coords) {
+    long cnt = 0;
+    for (long t = 0; t < T; t++)
+        for (int c = 0; c < n; c++)
+            if (mask[t * n + c]) coords[cnt++] = (uint16_t)(((t & 15) << 8) | c);
+    return cnt;
+}
+
 /* Sideband for one (b, h) stream: flagged chunks copied in (token, chunk)
  * order; tile_off[i] = number of flagged chunks before token 16*i. Returns the count. */
 long orc_pack_sideband(const void *x, const uint8_t *mask, int dt, long T, int n, void *sideband,

@@ -101,6 +101,7 @@ def test_flags_and_sideband_match_oracle(S, b_r, dn, d_h):
                 assert int(pt.sb_count[b, h]) == cnt
                 assert bit_equal(pt.sideband[b, h, :cnt], sb)
                 assert torch.equal(pt.sb_tile_off[b, h, :toff.numel()].cpu(), toff)
+                assert torch.equal(pt.sb_coord[b, h, :cnt].cpu(), CO.pack_coords(want["mask"][b, h]))
         assert bit_equal(ops.dequant_packed(pt, T, mode=1), want["out"])
         dense = CO.dequant(want["idx"], want["rq"], want["r_max"], Jc, pt.qmax).view(B, H, T, n, 4)
         dense = torch.where(want["mask"].unsqueeze(-1), x.view(B, H, T, n, 4), dense).reshape(B, H, T, d_h)
@@ -131,6 +132,7 @@ def test_bulk_append_compaction_then_more_appends(dn, d_h):
             assert int(cache.K.sb_count[b, h]) == cnt and cnt > 0
             assert bit_equal(cache.K.sideband[b, h, :cnt], sb)
             assert torch.equal(cache.K.sb_tile_off[b, h, :toff.numel()].cpu(), toff)
+            assert torch.equal(cache.K.sb_coord[b, h, :cnt].cpu(), CO.pack_coords(masks[b, h]))
 
 
 def test_decode_appends_keep_sideband_consistent():
