@@ -197,7 +197,7 @@ def test_decode_loop_with_append_config4_shape():
         sub = w.new_cache(1, Tmax, d_h, dt, 0, sideband_frac=0.25)
         w.append(sub, k_all[b:b + 1, :, :L0].to(DEV), v_all[b:b + 1, :, :L0].to(DEV), 0)
         for dst, src in ((cache.K, sub.K), (cache.V, sub.V)):
-            for name in ("main", "aux", "scale", "flags", "sideband", "sb_tile_off", "sb_count"):
+            for name in ("main", "aux", "scale", "flags", "sideband", "sb_tile_off", "sb_count", "sb_coord"):
                 getattr(dst, name)[b] = getattr(src, name)[0]
         dk, dv = oracle_dense(k_all[b:b + 1, :, :L0].contiguous(), Jk), oracle_dense(v_all[b:b + 1, :, :L0].contiguous(), Jv)
         ref_k[b, :, :L0], ref_kx[b, :, :L0] = dk[0][0], dk[1][0]
@@ -271,3 +271,38 @@ def test_config3_and_5_full_size_properties(cfg):
         assert (o.float() - O.float()).abs().max().item() < 1e-3 * scale
     og = hqmq.fused_attention_packed(Q, cache, force_generic=True)
     assert (og.float() - O.float()).abs().max().item() < 1e-3 * scale
+
+
+@pytest.mark.parametrize("d_h,Tq,hot,dn", [(64, 1, (2, 5), "fp16"), (64, 144, (2, 5), "fp16"), (64, 1, (0, 1, 2, 3), "bf16"),
+                                            (128, 1, (0, 1, 2, 8, 30), "fp16"), (128, 9, (3, 17), "bf16")])
+def test_clustered_outlier_channels(d_h, Tq, hot, dn):
+    """Outlier *channels*: the same chunk positions are flagged in most tokens (up to 25 % of all chunks, several per
+    lane and more than 64 per half-step), decode and chunked prefill; specialised and layout-generic kernels
+    against dense fp32 attention over the dequantized cache."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = DT[dn]
+    B, Hq, Hkv, T = 2, 8, 2, 150
+    g = torch.Generator().manual_seed(3)
+    k, v = torch.randn(B, Hkv, T, d_h, generator=g), torch.randn(B, Hkv, T, d_h, generator=g)
+    for c in hot:
+        k[..., 4 * c:4 * c + 4] *= 12.0
+        v[..., 4 * c:4 * c + 4] *= 12.0
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    cache = w.new_cache(B, T, d_h, dt, 0, sideband_frac=0.5)
+    w.append(cache, k.to(dt).to(DEV), v.to(dt).to(DEV), 0)
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    assert float(cache.K.sb_count.sum()) / (B * Hkv * T * d_h / 4) > 0.02
+    Q = torch.randn(B, Hq, Tq, d_h, generator=g).to(dt).to(DEV)
+    off = T - Tq
+    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    mask = torch.arange(T, device=DEV).view(1, 1, 1, T) <= (torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off)
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
+    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))     # bf16: the output's own rounding
+    for generic in (False, True):
+        for ns in (0, 3):
+            O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, force_generic=generic, n_splits=ns)
+            assert (O.float() - ref).abs().max().item() < tol, (generic, ns)
