@@ -103,6 +103,9 @@ __device__ __forceinline__ float scaled(float acc, uint32_t pair, int hi, float 
 // The dynamic LDS block is the kernel's only LDS, so it starts at LDS address 0: the K table sits at byte 0,
 // the V table at kVTabOffset, and a gather addresses them with idx * 8 (+ the instruction's immediate offset).
 constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
+constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
 
 template <int TAB_OFF>
 __device__ __forceinline__ half4 gather8(uint32_t byte_addr) {
@@ -127,6 +130,26 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
             a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
             a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
+        }
+    } else if constexpr (MB == 12 && AB == 1 && IB == 10 && CPL == 8) {
+        // s24_r3: eight 12-bit fields (idx in the low 10 bits, the low two radius bits above) in three dwords
+        // and one aux byte with the eight high radius bits.  The aux byte indexes a 256-entry LDS table whose row
+        // holds, per pair of chunks, the two high radius bits at bits 2 and 18 and the 0x6400 fp16 magic.
+        const uint4v ax = *(lds_u4_ptr)(uintptr_t)(kAuxTabOffset + (aux & 0xffu) * 16u);
+        const uint32_t axs[4] = {ax[0], ax[1], ax[2], ax[3]};
+        const uint32_t w0 = w[0], w1 = w[1], w2 = w[2];
+        constexpr uint32_t M = 0x1ff8u;
+        const uint32_t ad[8] = {(w0 << 3) & M, (w0 >> 9) & M, __builtin_amdgcn_alignbit(w1, w0, 21) & M, (w1 >> 1) & M,
+                                (w1 >> 13) & M, __builtin_amdgcn_alignbit(w2, w1, 25) & M, (w2 >> 5) & M, (w2 >> 17) & M};
+        const uint32_t lo2[8] = {__builtin_amdgcn_ubfe(w0, 10, 2), __builtin_amdgcn_ubfe(w0, 22, 2), __builtin_amdgcn_ubfe(w1, 2, 2),
+                                 __builtin_amdgcn_ubfe(w1, 14, 2), __builtin_amdgcn_ubfe(w1, 26, 2), __builtin_amdgcn_ubfe(w2, 6, 2),
+                                 __builtin_amdgcn_ubfe(w2, 18, 2), w2 >> 30};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t t = (lo2[2 * i] | (lo2[2 * i + 1] << 16)) | axs[i];
+            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
+            a[2 * i] = gather8<TAB_OFF>(ad[2 * i]) * r[0];
+            a[2 * i + 1] = gather8<TAB_OFF>(ad[2 * i + 1]) * r[1];
         }
     } else {
 #pragma unroll
@@ -313,6 +336,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     if (max(Kk, Kv) > FU * NT)
         fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
+    if constexpr (MB == 12 && AB == 1 && IB == 10) {
+        if (threadIdx.x < 256) {
+            const uint32_t b8 = threadIdx.x;
+            uint32_t row[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) row[i] = (((b8 >> (2 * i)) & 1u) << 2) | (((b8 >> (2 * i + 1)) & 1u) << 18) | 0x64006400u;
+            lds_tab[kAuxTabOffset / 8 + 2 * b8] = uint2{row[0], row[1]};
+            lds_tab[kAuxTabOffset / 8 + 2 * b8 + 1] = uint2{row[2], row[3]};
+        }
+    }
     __syncthreads();
 
     // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
@@ -579,6 +612,7 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     *handled = true;
     if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st);
     if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st);
     *handled = false;
