@@ -187,3 +187,19 @@ def test_algorithmic_bytes_per_token():
         n = d_h // 4
         assert (n * mb + 7) // 8 + (n * ab + 7) // 8 + 2 == want
         assert n * (ib + b_r) // 8 + 2 == want
+
+
+def test_memory_table_uses_packed_layout():
+    """The memory table counts what the planes store: whole bits per code, scale, and with Med3x flags + sideband."""
+    from hqmq_amd import memory_table as MT
+    assert [MT.row_bytes(128, S, b) for S, b in MT.CONFIGS] == [54, 58, 62, 66, 70, 78]
+    assert MT.row_bytes(64, 96, 4) == 34
+    assert MT.row_bytes(128, 192, 6, med3x=0.02) == 78 + 4 + 0.02 * 32 * 8
+    rows = MT.table()
+    r = next(x for x in rows if x["model"] == "Llama-3-8B" and x["seq_len"] == 32768)
+    assert r["fp16_MB"] == 2 * 32 * 8 * 32768 * 128 * 2 / 1e6
+    assert abs(r["hqmq_s96_r4_MB"] - 2 * 32 * 8 * 32768 * 66 / 1e6) < 1e-9
+    # never below the reference's analytic figure (fractional log2 bits), and within 6 % of it
+    for S, b in MT.CONFIGS:
+        k = f"hqmq_s{S}_r{b}"
+        assert r[k + "_analytic_MB"] <= r[k + "_MB"] <= 1.06 * r[k + "_analytic_MB"]
