@@ -199,7 +199,7 @@ def test_memory_table_uses_packed_layout():
     r = next(x for x in rows if x["model"] == "Llama-3-8B" and x["seq_len"] == 32768)
     assert r["fp16_MB"] == 2 * 32 * 8 * 32768 * 128 * 2 / 1e6
     assert abs(r["hqmq_s96_r4_MB"] - 2 * 32 * 8 * 32768 * 66 / 1e6) < 1e-9
-    # never below the reference's analytic figure (fractional log2 bits), and within 6 % of it
+    # never below the reference's analytic figure (fractional log2 bits), and within 8 % of it
     for S, b in MT.CONFIGS:
         k = f"hqmq_s{S}_r{b}"
-        assert r[k + "_analytic_MB"] <= r[k + "_MB"] <= 1.06 * r[k + "_analytic_MB"]
+        assert r[k + "_analytic_MB"] <= r[k + "_MB"] <= 1.08 * r[k + "_analytic_MB"]
