@@ -105,6 +105,18 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
     """
     if T_kv is None:
         T_kv = cache.K.t_cap if kv_lens is not None else cache.K.length
+    d, d_store = Q.shape[-1], cache.K.d_head
+    if d < d_store and d == cache.K.d_head_orig:
+        # a cache of zero-padded heads (PaddedHQMQ): pad Q the same way, keep the scale of the real head size
+        if softmax_scale is None:
+            softmax_scale = d ** -0.5
+        O = ops.attn_fwd(torch.nn.functional.pad(Q, (0, d_store - d)), cache.K, cache.V, T_kv, kv_lens=kv_lens, causal=causal,
+                         causal_offset=causal_offset, softmax_scale=softmax_scale, n_splits=n_splits,
+                         force_generic=force_generic)[..., :d]
+        if out is not None:
+            out.copy_(O)
+            return out
+        return O.contiguous()
     return ops.attn_fwd(Q, cache.K, cache.V, T_kv, kv_lens=kv_lens, causal=causal, causal_offset=causal_offset,
                         softmax_scale=softmax_scale, n_splits=n_splits, out=out, force_generic=force_generic)
 

@@ -395,11 +395,11 @@ extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv
 extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,
                                  int64_t o_sb, int64_t o_sh, int64_t o_st, void *stream) {
     if (!workspace || !O) return HQMQ_ERR_NULL;
-    if (B < 1 || H_q < 1 || T_q < 1 || d_h < 4 || d_h > 256 || (d_h & (d_h - 1)) || n_splits < 1 || n_splits > 8192) return HQMQ_ERR_SHAPE;
+    if (B < 1 || H_q < 1 || T_q < 1 || d_h < 4 || d_h > 256 || (d_h & 3) || n_splits < 1 || n_splits > 8192) return HQMQ_ERR_SHAPE;
     if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(d_h < 64 ? 64 : d_h), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3((d_h + 63) / 64 * 64), 0, (hipStream_t)stream,
                        (const float *)workspace, O,
                        dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
@@ -419,7 +419,9 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if ((int64_t)a->B * a->H_kv > 65535) return HQMQ_ERR_SHAPE;
     if (a->t_cap < a->T_kv || a->t_cap < 1) return HQMQ_ERR_SHAPE;
     const int n = a->n_chunks;
-    if (n < 4 || n > 64 || (n & (n - 1)) || a->qmax < 1) return HQMQ_ERR_SHAPE;  // d_h in {16, 32, 64, 128, 256}
+    // d_h in {16, 32, 64, 128, 256} and, for heads padded from sizes such as 80 or 160, {80, 160}
+    if (n < 4 || n > 64 || (n & 3) || a->qmax < 1) return HQMQ_ERR_SHAPE;
+    if ((n & (n - 1)) && n != 20 && n != 40) return HQMQ_ERR_SHAPE;
     if (a->idx_bits < 1 || a->idx_bits > 16 || a->aux_bits < 0 || a->aux_bits > 8) return HQMQ_ERR_LAYOUT;
     if ((a->K.flag_plane != nullptr) != (a->V.flag_plane != nullptr)) return HQMQ_ERR_NULL;
     const bool flags = a->K.flag_plane != nullptr;
@@ -478,7 +480,9 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
         case 1: rc = launch_attn_mb<1>(p, a->main_bits, flags, grid, shmem, st); break;
         case 2: rc = launch_attn_mb<2>(p, a->main_bits, flags, grid, shmem, st); break;
         case 4: rc = launch_attn_mb<4>(p, a->main_bits, flags, grid, shmem, st); break;
+        case 5: rc = launch_attn_mb<5>(p, a->main_bits, flags, grid, shmem, st); break;
         case 8: rc = launch_attn_mb<8>(p, a->main_bits, flags, grid, shmem, st); break;
+        case 10: rc = launch_attn_mb<10>(p, a->main_bits, flags, grid, shmem, st); break;
         case 16: rc = launch_attn_mb<16>(p, a->main_bits, flags, grid, shmem, st); break;
         default: return HQMQ_ERR_SHAPE;
     }

@@ -374,8 +374,12 @@ extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
     if (24 * a->secondary_size > 65535) return HQMQ_ERR_SHAPE;  // candidate lists hold 16-bit indices
     const bool packed = a->main_plane || a->aux_plane || a->flag_plane || a->scale_plane;
     if (packed) {
-        if (a->main_bits != mb || a->aux_bits != ab) return HQMQ_ERR_LAYOUT;
-        if (ab && a->main_plane && !a->aux_plane) return HQMQ_ERR_NULL;
+        // the layout rule's widths, or any wider split that still holds idx_bits + radius_bits (16-bit rows for heads
+        // whose lanes would otherwise get an odd number of 12-bit codes)
+        if (a->main_bits < 1 || a->main_bits > 16 || a->aux_bits < 0 || a->aux_bits > 8 ||
+            a->main_bits + a->aux_bits < ib + a->radius_bits)
+            return HQMQ_ERR_LAYOUT;
+        if (a->aux_bits && a->main_plane && !a->aux_plane) return HQMQ_ERR_NULL;
         if (a->t_cap < 1 || a->t_off < 0) return HQMQ_ERR_SHAPE;
         if (!a->pos && (int64_t)a->t_off + a->T > a->t_cap) return HQMQ_ERR_SHAPE;
         if (a->flag_plane && !a->thr) return HQMQ_ERR_NULL;
@@ -388,7 +392,7 @@ extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
     p.thr = a->thr; p.mask_out = a->mask_out;
     p.main_plane = a->main_plane; p.aux_plane = a->aux_plane; p.flag_plane = a->flag_plane;
     p.scale_plane = a->scale_plane; p.t_cap = a->t_cap; p.t_off = a->t_off; p.pos = a->pos;
-    p.idx_bits = ib; p.main_bits = mb; p.aux_bits = ab;
+    p.idx_bits = ib; p.main_bits = packed ? a->main_bits : mb; p.aux_bits = packed ? a->aux_bits : ab;
     p.tokens_per_block = kQThreads / a->n_chunks;
     p.stats = a->stats;
     hipStream_t st = (hipStream_t)stream;

@@ -31,6 +31,7 @@ class PackedTensor:
         if d_head % 4:
             raise ValueError(f"d_head={d_head} not divisible by 4")
         self.B, self.H, self.d_head, self.n = B, H, d_head, d_head // 4
+        self.d_head_orig = d_head            # smaller for zero-padded heads (PaddedHQMQ): what Q and O carry
         self.t_cap = _round_up(max(t_cap, 1), T_ALIGN)
         self.secondary_size, self.radius_bits = secondary_size, radius_bits
         self.qmax = (1 << radius_bits) - 1

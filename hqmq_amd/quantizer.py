@@ -397,3 +397,42 @@ class PaddedHQMQQuantizer(KVQuantizer):
     @property
     def name(self):
         return f"PaddedHQMQ_d{self.d_head_orig}to{self.d_head_padded}_{self.inner.name}"
+
+    # ---- packed cache: the head is zero-padded to a size the attention kernels take ----
+    _ATTN_DIMS = (16, 32, 64, 80, 128, 160, 256)
+
+    @property
+    def d_head_stored(self) -> int:
+        """Head size of the packed planes: the smallest the attention kernels support that holds d_head.
+        The extra chunks are all-zero, quantize to radius code 0 and decode to exactly 0."""
+        for d in self._ATTN_DIMS:
+            if d >= self.d_head_padded:
+                return d
+        raise L.HqmqError(f"d_head={self.d_head_orig} is beyond the attention kernels' 256")
+
+    def _pad(self, x: torch.Tensor) -> torch.Tensor:
+        d = x.shape[-1]
+        if d == self.d_head_stored:
+            return x
+        assert d in (self.d_head_orig, self.d_head_padded), f"Expected d_head={self.d_head_orig}, got {d}"
+        return torch.nn.functional.pad(x, (0, self.d_head_stored - d))
+
+    def new_cache(self, batch: int, max_tokens: int, dtype: torch.dtype, layer_idx: int) -> PackedKV:
+        """An empty bit-packed cache of d_head_stored-wide heads (12-bit code rows need an even number of chunks
+        per lane; where the head does not give that, codes are stored 16 bits wide)."""
+        inner, d = self.inner, self.d_head_stored
+        inner._check_supported()
+        idx_bits, main_bits, aux_bits = L.layout_bits(inner.secondary_size, inner.radius_bits)
+        layout = None
+        if main_bits == 12 and (d // 16) % 2:
+            layout = (idx_bits, 16, max(0, idx_bits + inner.radius_bits - 16))
+        dev = inner.secondary_raw.device
+        ref = torch.empty(0, dtype=dtype, device=dev)
+        mk = lambda kv: PackedTensor(batch, inner.n_heads, max_tokens, d, inner.secondary_size, inner.radius_bits, dtype, dev,
+                                     joint=inner._joint_and_slack(layer_idx, kv, ref)[0], layout=layout)
+        kv = PackedKV(mk(0), mk(1))
+        kv.K.d_head_orig = kv.V.d_head_orig = self.d_head_orig
+        return kv
+
+    def append(self, cache: PackedKV, k: torch.Tensor, v: torch.Tensor, layer_idx: int, pos=None) -> None:
+        self.inner.append(cache, self._pad(k), self._pad(v), layer_idx, pos=pos)

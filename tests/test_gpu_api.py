@@ -3,6 +3,7 @@ import pytest
 import torch
 
 pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
+DEV = "cuda"
 
 
 def test_quantize_on_gpu():
@@ -75,3 +76,32 @@ def test_native_library_is_what_ran():
     so = str(L.library_path())
     with open("/proc/self/maps") as f:
         assert any(so in line for line in f)
+
+
+@pytest.mark.parametrize("d_head,S,b_r", [(80, 96, 4), (70, 24, 3), (160, 24, 4), (100, 96, 4)])
+def test_padded_quantizer_packed_path(d_head, S, b_r):
+    """PaddedHQMQ on the packed path: heads that are no multiple of 4 (or no size the attention kernels take) are
+    zero-padded into the planes; the planes decode to the fake-quant tensor bit for bit and fused attention equals
+    dense attention over it."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.float16
+    B, Hq, Hkv, T = 2, 8, 2, 200
+    q = hqmq.PaddedHQMQ(n_layers=1, n_heads=Hkv, d_head=d_head, secondary_size=S, radius_bits=b_r, device=DEV)
+    g = torch.Generator().manual_seed(d_head)
+    k, v = torch.randn(B, Hkv, T, d_head, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_head, generator=g).to(dt).to(DEV)
+    cache = q.new_cache(B, T, dt, 0)
+    q.append(cache, k[:, :, :150], v[:, :, :150], 0)
+    q.append(cache, k[:, :, 150:], v[:, :, 150:], 0)
+    assert cache.K.d_head == q.d_head_stored >= d_head
+    kq, vq = q.quantize_K(k, 0), q.quantize_V(v, 0)
+    dk = ops.dequant_packed(cache.K, T, mode=1)
+    assert torch.equal(dk[..., :d_head].contiguous().view(torch.int16), kq.contiguous().view(torch.int16))
+    assert int(dk[..., q.d_head_padded:].abs().sum()) == 0          # whole padding chunks decode to exactly zero
+    Q = torch.randn(B, Hq, 1, d_head, generator=g).to(dt).to(DEV)
+    O = hqmq.fused_attention_packed(Q, cache)
+    Kd = ops.dequant_packed(cache.K, T, 0)[..., :d_head].float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0)[..., :d_head].float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_head ** -0.5
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
+    assert O.shape == Q.shape and (O.float() - ref).abs().max().item() < 2e-3
