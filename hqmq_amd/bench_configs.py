@@ -144,6 +144,17 @@ def run(cfg, steps):
             hqmq.fused_attention_packed(Q, cache, kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out)
         res["us_per_step_with_append"] = round(event_us(step, steps), 2)
         res["us_append_only"] = round(event_us(lambda: w.append(cache, k1, v1, 0, pos=pos), steps), 2)
+        # the same step replayed from a HIP graph: what the GPU needs once the ten small launches of an append are
+        # not paced by the host (every kernel of the path is capturable: no allocation, no memset, no sync)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        res["us_per_step_with_append_graph"] = round(event_us(graph.replay, steps), 2)
     print(json.dumps(res), flush=True)
 
 

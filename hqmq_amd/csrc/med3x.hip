@@ -110,7 +110,8 @@ __global__ __launch_bounds__(1024) void med_hist_lds_kernel(const typename D::st
 }
 
 // Finds the bins holding 0-based ranks r_lo <= r_hi in a histogram of `bins` counters.
-// One block of 1024 threads; results through shared memory.
+// One block of 1024 threads: every thread sums its bins/1024 consecutive counters, a block-wide scan gives each
+// thread the rank range of its segment, and the thread whose range holds a wanted rank walks its own segment.
 __device__ void select_two(const uint32_t *hist, int bins, int64_t r_lo, int64_t r_hi, uint32_t *key_lo, uint32_t *key_hi,
                            int64_t *in_lo, int64_t *in_hi) {
     __shared__ unsigned long long part[1024];
@@ -120,26 +121,29 @@ __device__ void select_two(const uint32_t *hist, int bins, int64_t r_lo, int64_t
     unsigned long long s = 0;
     for (int i = 0; i < per; i++) s += hist[threadIdx.x * per + i];
     part[threadIdx.x] = s;
+    if (threadIdx.x < 2) { res[threadIdx.x] = (uint32_t)(bins - 1); resr[threadIdx.x] = 0; }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned long long run = 0;
-        int which = 0;
-        const int64_t want[2] = {r_lo, r_hi};
-        for (int i = 0; i < 1024 && which < 2; i++) {
-            while (which < 2 && (unsigned long long)want[which] < run + part[i]) {
-                unsigned long long r2 = run;
-                for (int j = 0; j < per; j++) {
-                    const uint32_t cnt = hist[i * per + j];
-                    if ((unsigned long long)want[which] < r2 + cnt) {
-                        res[which] = (uint32_t)(i * per + j);
-                        resr[which] = (long long)((unsigned long long)want[which] - r2);
-                        break;
-                    }
-                    r2 += cnt;
+    for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scan
+        const unsigned long long v = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    const unsigned long long incl = part[threadIdx.x], excl = incl - s;
+    const int64_t want[2] = {r_lo, r_hi};
+    for (int which = 0; which < 2; which++) {
+        const unsigned long long w = (unsigned long long)want[which];
+        if (w >= excl && w < incl) {
+            unsigned long long r2 = excl;
+            for (int j = 0; j < per; j++) {
+                const uint32_t cnt = hist[threadIdx.x * per + j];
+                if (w < r2 + cnt) {
+                    res[which] = (uint32_t)(threadIdx.x * per + j);
+                    resr[which] = (long long)(w - r2);
+                    break;
                 }
-                which++;
+                r2 += cnt;
             }
-            run += part[i];
         }
     }
     __syncthreads();
