@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--context 32768] [--n-splits 0]
 
-A step is one fused decode-attention pass of one layer over the compressed cache of BASELINE config 2
+A step is one fused decode-attention pass of one layer over the compressed cache of benchmark config 2
 (Llama-3-8B shape: 32 query / 8 KV heads, d_h = 128, batch 1, s96_r4, fp16, context 32768, one query
 token, causal=False).  Inputs (packed cache, query) are resident in HBM before the timed region.  The K
 timed steps are captured in one HIP graph and replayed once, bracketed by torch.cuda.synchronize().

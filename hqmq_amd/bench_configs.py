@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Full-size runs of BASELINE configs 3, 4 and 5 on one GPU (config 2 is bench.py's default workload).
+"""Full-size runs of benchmark configs 3, 4 and 5 on one GPU (config 2 is bench.py's default workload).
 
     python -m hqmq_amd.bench_configs [--configs 3 4 5] [--steps 50]
 

@@ -1,4 +1,4 @@
-// Attention kernels specialised at compile time for the layouts the BASELINE shapes use:
+// Attention kernels specialised at compile time for the layouts of the benchmark shapes:
 // d_h = 64 / 128, fp16 or bf16 caches, codes of 16+0 (s96_r4), 12+1 (s24_r3) or 16+3 (s192_r6) bits.
 //
 // Lane mapping (one wavefront, one 16-token tile): lane = 16 * grp + col decodes the CPL = d_h / 16 chunks

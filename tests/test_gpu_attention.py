@@ -128,7 +128,7 @@ def test_attention_matches_dense_oracle(case):
 
 
 def test_torch_sdpa_agrees_on_the_same_cache():
-    """Dense SDPA on the GPU over the dequantized cache (what BASELINE config 2 names as the check)."""
+    """Dense SDPA on the GPU over the dequantized cache (the check benchmark config 2 asks for)."""
     import hqmq
     from hqmq_amd import ops
     dt = torch.float16
@@ -144,7 +144,7 @@ def test_torch_sdpa_agrees_on_the_same_cache():
 
 @pytest.mark.parametrize("T", [4096, 32768])
 def test_config2_full_size_properties(T):
-    """BASELINE config 2 at full size (32 / 8 heads, d_h=128, s96_r4, fp16, one query token):
+    """Benchmark config 2 at full size (32 / 8 heads, d_h=128, s96_r4, fp16, one query token):
     split invariance, zero padding rows ignored, agreement with dense fp32 attention on the GPU, 2e-3 bound."""
     import hqmq
     from hqmq_amd import ops
@@ -240,7 +240,7 @@ def test_argument_checks():
 
 @pytest.mark.parametrize("cfg", [3, 5])
 def test_config3_and_5_full_size_properties(cfg):
-    """BASELINE configs 3 (28/4 heads, batch 8, 32k, s192_r6 + Med3x, fp16, 2 % of K chunks x50-200) and
+    """Benchmark configs 3 (28/4 heads, batch 8, 32k, s192_r6 + Med3x, fp16, 2 % of K chunks x50-200) and
     5 (64/8 heads, d_h 64, batch 4, 131072, s96_r4 + Med3x, bf16, 1 % of chunks x100) at full size: agreement with
     dense fp32 attention over the dequantized cache, split invariance, and the specialised kernel against the
     layout-generic one.  Outputs reach |O| ~ 4 (config 3) and ~ 350 (config 5), so bounds are relative to that."""

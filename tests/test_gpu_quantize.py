@@ -102,7 +102,7 @@ def test_strided_input_and_error_paths():
 
 
 def test_full_size_config1_round_trip():
-    """BASELINE config 1 at full size (8 KV heads, d_h=128, T=2048, s24_r3 + Med3x, fp16): codes, scales,
+    """Benchmark config 1 at full size (8 KV heads, d_h=128, T=2048, s24_r3 + Med3x, fp16): codes, scales,
     mask and the fake-quant tensor bit-exact against the oracle; MSE reported."""
     import hqmq
     dt = torch.float16
