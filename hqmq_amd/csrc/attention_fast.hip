@@ -106,6 +106,7 @@ constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords 
 constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
+typedef const uint32_t __attribute__((address_space(3))) *lds_u1_ptr;
 
 template <int TAB_OFF>
 __device__ __forceinline__ half4 gather8(uint32_t byte_addr) {
@@ -127,6 +128,20 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
             const uint32_t t = ((w[i] >> idx_bits) & rq2) | 0x64006400u;
+            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
+            a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
+            a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
+        }
+    } else if constexpr (MB == 16 && AB == 3 && IB == 13) {
+        // s192_r6: idx (13 bits) and the low three radius bits in the 16-bit main field, the high three in the aux
+        // row.  Six aux bits (two chunks) index a 64-entry LDS table holding them at bits 3..5 and 19..21 together
+        // with the 0x6400 fp16 magic.
+        constexpr uint32_t im2 = 0x1fff1fffu;
+#pragma unroll
+        for (int i = 0; i < CPL / 2; i++) {
+            const uint32_t ix = w[i] & im2;
+            const uint32_t hi = *(lds_u1_ptr)(uintptr_t)(kAuxTabOffset + ((aux >> (6 * i)) & 63u) * 4u);
+            const uint32_t t = ((w[i] >> 13) & 0x00070007u) | hi;
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
             a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
             a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
@@ -336,6 +351,12 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     if (max(Kk, Kv) > FU * NT)
         fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
+    if constexpr (MB == 16 && AB == 3 && IB == 13) {
+        if (threadIdx.x < 64) {
+            const uint32_t b6 = threadIdx.x;
+            reinterpret_cast<uint32_t *>(lds_tab)[kAuxTabOffset / 4 + b6] = ((b6 & 7u) << 3) | ((b6 >> 3) << 19) | 0x64006400u;
+        }
+    }
     if constexpr (MB == 12 && AB == 1 && IB == 10) {
         if (threadIdx.x < 256) {
             const uint32_t b8 = threadIdx.x;
@@ -614,6 +635,7 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st);
     *handled = false;
     return HQMQ_OK;
