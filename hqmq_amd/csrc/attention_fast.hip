@@ -421,7 +421,13 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
                     so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(m0 ? val : zero_h4, m1 ? val : zero_h4), qf[jj], so, 0, 0, 0);
             }
         };
-        one(o.fl ? __builtin_ctz(o.fl) : 255, o.v0);
+        {   // the first flagged chunk of every lane: straight-line, one MFMA per pair of chunk positions
+            const int j0 = o.fl ? __builtin_ctz(o.fl) : 255;
+#pragma unroll
+            for (int jj = 0; jj < CPL / 2; jj++)
+                so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(j0 == 2 * jj ? o.v0 : zero_h4, j0 == 2 * jj + 1 ? o.v0 : zero_h4),
+                                                            qf[jj], so, 0, 0, 0);
+        }
         const uint32_t r1 = o.fl & (o.fl - 1u);
         if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
             one(r1 ? __builtin_ctz(r1) : 255, o.v1);
@@ -436,7 +442,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         }
     };
     // V side: the verbatim chunks, transposed, times the unscaled probabilities of the tile.
-    auto out_apply_v = [&](const OutPre &o, half4 pTo) {
+    auto out_apply_v = [&](const OutPre &o, half4 pTo) {      // second and further flagged chunks of a lane (rare)
         if (!o.any) return;
         auto one = [&](int jme, half4 val) {
 #pragma unroll
@@ -448,7 +454,6 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
                 }
             }
         };
-        one(o.fl ? __builtin_ctz(o.fl) : 255, o.v0);
         const uint32_t r1 = o.fl & (o.fl - 1u);
         if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
             one(r1 ? __builtin_ctz(r1) : 255, o.v1);
@@ -532,6 +537,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
         }
         if (FLAGS) {
+            if (oc[2].any || oc[3].any) {   // the first flagged chunk of every lane, both tiles in one 16x16x32 MFMA
+                const int j0 = oc[2].fl ? __builtin_ctz(oc[2].fl) : 255, j1 = oc[3].fl ? __builtin_ctz(oc[3].fl) : 255;
+                const half8 ppo = cat8(pTo[0], pTo[1]);
+#pragma unroll
+                for (int j = 0; j < CPL; j++) {
+                    const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(j0 == j ? oc[2].v0 : zero_h4, ident, zero4, 0, 0, 0);
+                    const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(j1 == j ? oc[3].v0 : zero_h4, ident, zero4, 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), ppo, acc[j], 0, 0, 0);
+                }
+            }
             out_apply_v(oc[2], pTo[0]);
             out_apply_v(oc[3], pTo[1]);
         }
