@@ -122,12 +122,15 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
     const int idx_bits = IB ? IB : idx_bits_rt;
     const uint32_t idx_mask = (1u << idx_bits) - 1u;
     if constexpr (MB == 16 && AB == 0) {
-        const uint32_t rq2 = (0xffffu >> idx_bits) * 0x00010001u;
+        // mask in a scalar register and magic in a vector register, so that (x & mask) | magic is one v_and_or_b32
+        uint32_t rq2 = (0xffffu >> idx_bits) * 0x00010001u, magic = 0x64006400u;
+        asm("" : "+s"(rq2));
+        asm("" : "+v"(magic));
         const uint32_t im2 = idx_mask * 0x00010001u;
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
-            const uint32_t t = ((w[i] >> idx_bits) & rq2) | 0x64006400u;
+            const uint32_t t = ((w[i] >> idx_bits) & rq2) | magic;
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
             a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
             a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
