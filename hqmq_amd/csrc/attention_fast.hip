@@ -113,6 +113,18 @@ __device__ __forceinline__ half4 gather8(uint32_t byte_addr) {
     return __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(byte_addr + TAB_OFF));
 }
 
+// Table byte address of the low (HI = 0) or high (HI = 1) 16-bit index of a masked pair: one shift that reads
+// a half of the register (the compiler's own lowering is a shift and an and).
+template <int HI>
+__device__ __forceinline__ uint32_t half_addr8(uint32_t pair) {
+    uint32_t r;
+    if constexpr (HI)
+        asm("v_lshlrev_b32_sdwa %0, 3, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1" : "=v"(r) : "v"(pair));
+    else
+        asm("v_lshlrev_b32_sdwa %0, 3, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0" : "=v"(r) : "v"(pair));
+    return r;
+}
+
 // Decodes the CPL chunks of one lane: gather from the LDS table, times the radius code.
 // 16+0 layout: the two radius codes of a dword become an fp16 pair with one shift, one and-or
 // (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract.  IB = idx_bits when known at compile
@@ -132,8 +144,8 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
             const uint32_t ix = w[i] & im2;
             const uint32_t t = ((w[i] >> idx_bits) & rq2) | magic;
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
-            a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
+            a[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix)) * r[0];
+            a[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix)) * r[1];
         }
     } else if constexpr (MB == 16 && AB == 3 && IB == 13) {
         // s192_r6: idx (13 bits) and the low three radius bits in the 16-bit main field, the high three in the aux
@@ -146,8 +158,8 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
             const uint32_t hi = *(lds_u1_ptr)(uintptr_t)(kAuxTabOffset + ((aux >> (6 * i)) & 63u) * 4u);
             const uint32_t t = ((w[i] >> 13) & 0x00070007u) | hi;
             const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = gather8<TAB_OFF>((ix & 0xffffu) << 3) * r[0];
-            a[2 * i + 1] = gather8<TAB_OFF>((ix >> 16) << 3) * r[1];
+            a[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix)) * r[0];
+            a[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix)) * r[1];
         }
     } else if constexpr (MB == 12 && AB == 1 && IB == 10 && CPL == 8) {
         // s24_r3: eight 12-bit fields (idx in the low 10 bits, the low two radius bits above) in three dwords
