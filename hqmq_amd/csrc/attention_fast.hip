@@ -60,11 +60,20 @@ struct HalfTile {
     uint32_t kaux[AB ? 2 : 1], vaux[AB ? 2 : 1];
     uint2 ks[2], vs[2];
 };
-// flag words of the same 32 tokens; they travel one half-step ahead of the codes, so that the sideband chunks
-// they point to can be requested a whole half-step before use
+// outlier bookkeeping of the same 32 tokens; it travels one half-step ahead of the codes, so that the sideband
+// chunks it points to can be requested a whole half-step before use
 struct FlagTile {
-    uint32_t kfl[2], vfl[2];   // flag bits of token `col` of tile u
-    int ksb[2], vsb[2];        // sideband slot of tile u's first flagged chunk
+    int koff[3];               // K: sideband entries [koff[u], koff[u + 1]) belong to tile u (wave-uniform)
+    uint32_t vfl[2];           // V: flag bits of token `col` of tile u
+    int vsb[2];                // V: sideband slot of tile u's first flagged chunk
+};
+// K outliers of one half-step, requested ahead: the first kKPre batches of eight sideband entries.  Lane
+// 16 * grp + col holds entries 2 * grp and 2 * grp + 1 of a batch (the same in all 16 lanes of a row).
+constexpr int kKPre = 2;
+struct KPre {
+    int off[3];
+    uint2 x[kKPre][2];         // verbatim chunks (raw bits of the cache dtype)
+    uint32_t cc[kKPre];        // their coordinates: (token & 15) << 8 | chunk, two 16-bit fields
 };
 // the unit of prefetch: NH half-tiles (64 tokens; 32 for the variants with outlier flags, which need the registers)
 template <int NW, int AB, bool FLAGS, int NH>
@@ -103,6 +112,7 @@ __device__ __forceinline__ float scaled(float acc, uint32_t pair, int hi, float 
 // The dynamic LDS block is the kernel's only LDS, so it starts at LDS address 0: the K table sits at byte 0,
 // the V table at kVTabOffset, and a gather addresses them with idx * 8 (+ the instruction's immediate offset).
 constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
+constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chunk][column] fp16 chunks, after the V table
 constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
@@ -275,6 +285,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const size_t plane_row0 = (size_t)bh * p.t_cap;
     constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8, frb = (n + 7) / 8;
     const int64_t tiles_cap = p.t_cap / kTile;
+    const int tiles_cap1 = (int)tiles_cap - 1;
     const int idx_bits = p.idx_bits;
     const uint16_t *ks_plane = (const uint16_t *)p.Kc.scale_plane + b * p.Kc.ssb + hkv * p.Kc.ssh;
     const uint16_t *vs_plane = (const uint16_t *)p.Vc.scale_plane + b * p.Vc.ssb + hkv * p.Vc.ssh;
@@ -282,12 +293,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const uint8_t *v_rows = p.Vc.main_plane + plane_row0 * mrb;
     const uint8_t *ka_rows = AB ? p.Kc.aux_plane + plane_row0 * arb : nullptr;
     const uint8_t *va_rows = AB ? p.Vc.aux_plane + plane_row0 * arb : nullptr;
-    const uint8_t *kf_rows = FLAGS ? p.Kc.flag_plane + plane_row0 * frb : nullptr;
     const uint8_t *vf_rows = FLAGS ? p.Vc.flag_plane + plane_row0 * frb : nullptr;
     const int32_t *k_toff = FLAGS ? p.Kc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
     const int32_t *v_toff = FLAGS ? p.Vc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
     const uint32_t main_off = (uint32_t)(col * mrb + grp * NB), aux_off = (uint32_t)(col * arb + grp * ABYTES);
     const uint32_t flag_off = (uint32_t)(col * frb), scale_off = (uint32_t)(4 * grp);
+    const int k_count = FLAGS ? (int)min((int64_t)max(p.Kc.sb_count[bh], 0), p.Kc.sb_cap) : 0;
+    const char *k_side = FLAGS ? (const char *)p.Kc.sideband + (size_t)bh * p.Kc.sb_cap * 8 : nullptr;
+    const char *v_side = FLAGS ? (const char *)p.Vc.sideband + (size_t)bh * p.Vc.sb_cap * 8 : nullptr;
+    const char *k_coord = FLAGS ? (const char *)p.Kc.sb_coord + (size_t)bh * p.Kc.sb_cap * 2 : nullptr;
+    const uint32_t k_cap1 = FLAGS ? (uint32_t)(p.Kc.sb_cap - 1) : 0u, v_cap1 = FLAGS ? (uint32_t)(p.Vc.sb_cap - 1) : 0u;
 
     auto load_super = [&](int t0, FastTile<NW, AB, FLAGS, NH> &s) {
         // in the order the half-steps consume them: K, then V, of tokens 0..31, then the same of tokens 32..63
@@ -325,10 +340,14 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     auto load_flags = [&](int th, FlagTile &f) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            f.kfl[u] = load_small<frb>(kf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
             f.vfl[u] = load_small<frb>(vf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
-            f.ksb[u] = k_toff[(th >> 4) + u];
             f.vsb[u] = v_toff[(th >> 4) + u];
+        }
+        // tiles not written yet hold INT32_MAX, and so does the slot after the last tile: the count bounds them
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const int ti = (th >> 4) + i, v = k_toff[min(ti, tiles_cap1)];
+            f.koff[i] = min(ti <= tiles_cap1 ? v : 0x7fffffff, k_count);
         }
     };
 
@@ -366,6 +385,15 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     if (max(Kk, Kv) > FU * NT)
         fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
+    if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
+#pragma unroll
+        for (int jj = 0; jj < CPL / 2; jj++) {
+            const uint4v q8 = __builtin_bit_cast(uint4v, qf[jj]);
+            const int c0 = grp * CPL + 2 * jj;
+            lds_tab[kQOffset / 8 + c0 * 16 + col] = uint2{q8[0], q8[1]};
+            lds_tab[kQOffset / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
+        }
+    }
     if constexpr (MB == 16 && AB == 3 && IB == 13) {
         if (threadIdx.x < 64) {
             const uint32_t b6 = threadIdx.x;
@@ -411,49 +439,60 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         int slot;           // sideband slot of its first flagged chunk
         half4 v0, v1;       // its first two flagged chunks (requested early; more are rare and loaded on demand)
     };
-    auto out_issue = [&](const PackedDev &pc, uint32_t fw, int tile_off, OutPre &o) {
+    // Every load of the loop is issued unconditionally (clamped addresses): a load inside a branch would make the
+    // compiler's wait counts assume it was not issued, and the waits would then cover the next tile's prefetch.
+    auto out_issue = [&](const char *side, uint32_t cap1, uint32_t fw, int tile_off, OutPre &o) {
         o.any = __builtin_amdgcn_ballot_w64(fw != 0) != 0;
-        o.fl = 0;
-        o.slot = 0;
-        o.v0 = zero_h4;
-        o.v1 = zero_h4;
-        if (o.any) {
-            lane_flags(fw, tile_off, o.fl, o.slot);
-            const uint32_t r1 = o.fl & (o.fl - 1u);
-            if (o.fl) o.v0 = outlier_chunk(pc, DT, bh, o.slot);
-            if (r1) o.v1 = outlier_chunk(pc, DT, bh, o.slot + 1);
+        lane_flags(fw, (int)min((uint32_t)tile_off, cap1), o.fl, o.slot);
+        const uint32_t s0 = min((uint32_t)o.slot, cap1), s1 = min((uint32_t)o.slot + 1u, cap1);
+        o.v0 = chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(side + s0 * 8u));
+        o.v1 = chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(side + s1 * 8u));
+    };
+    // K side.  The sideband entries of a half-step are a contiguous range known from three tile offsets, so no
+    // flag is read: a batch of eight entries is the reduction dimension of one MFMA per tile,
+    //   so[token][column] += sum over entries e of the batch, i < 4:  [token(e) == token] x_e[i] * Q[column][4 chunk(e) + i],
+    // A = the lane's two entries where their token is the lane's row (else zero), B = the Q chunks they meet (LDS).
+    auto k_load = [&](int bs, uint2 (&x)[2], uint32_t &cc) {
+        // 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked at launch)
+        const uint32_t e0 = min((uint32_t)bs + 2u * (uint32_t)grp, k_cap1), e1 = min(e0 + 1u, k_cap1);
+        x[0] = *reinterpret_cast<const uint2 *>(k_side + e0 * 8u);
+        x[1] = *reinterpret_cast<const uint2 *>(k_side + e1 * 8u);
+        cc = (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e0 * 2u) | (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e1 * 2u) << 16;
+    };
+    auto k_issue = [&](const FlagTile &f, KPre &k) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) k.off[i] = f.koff[i];
+#pragma unroll
+        for (int bq = 0; bq < kKPre; bq++) {
+            k_load(k.off[0] + 8 * bq, k.x[bq], k.cc[bq]);
         }
     };
-    // Calls use(j, value) for every flagged chunk of the lane, j wave-uniform per call... the callee masks by lane.
-    // K side: the verbatim chunks times Q, accumulated unscaled in `so`.
-    auto out_apply_k = [&](const OutPre &o, float4v &so) {
-        if (!o.any) return;
-        auto one = [&](int jme, half4 val) {
+    auto k_batch = [&](const int (&off)[3], int bs, const uint2 (&x)[2], uint32_t cc, float4v (&so)[2]) {
+        const int e0 = bs + 2 * grp;
+        const uint32_t c0 = cc & (uint32_t)(n - 1), c1 = (cc >> 16) & (uint32_t)(n - 1);
+        const int r0 = (cc >> 8) & 15, r1 = (cc >> 24) & 15;
+        const half4 q0 = __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(kQOffset + c0 * 128u + (uint32_t)col * 8u));
+        const half4 q1 = __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(kQOffset + c1 * 128u + (uint32_t)col * 8u));
+        const half4 h0 = chunk_to_half<DT>(x[0]), h1 = chunk_to_half<DT>(x[1]);
+        const half8 qq = cat8(q0, q1);
 #pragma unroll
-            for (int jj = 0; jj < CPL / 2; jj++) {
-                const bool m0 = jme == 2 * jj, m1 = jme == 2 * jj + 1;
-                if (__builtin_amdgcn_ballot_w64(m0 || m1) != 0)
-                    so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(m0 ? val : zero_h4, m1 ? val : zero_h4), qf[jj], so, 0, 0, 0);
+        for (int u = 0; u < 2; u++) {
+            if (bs < off[u + 1] && bs + 8 > off[u]) {        // wave-uniform: the batch meets tile u
+                const bool v0 = e0 >= off[u] && e0 < off[u + 1] && r0 == col;
+                const bool v1 = e0 + 1 >= off[u] && e0 + 1 < off[u + 1] && r1 == col;
+                so[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(v0 ? h0 : zero_h4, v1 ? h1 : zero_h4), qq, so[u], 0, 0, 0);
             }
-        };
-        {   // the first flagged chunk of every lane: straight-line, one MFMA per pair of chunk positions
-            const int j0 = o.fl ? __builtin_ctz(o.fl) : 255;
-#pragma unroll
-            for (int jj = 0; jj < CPL / 2; jj++)
-                so = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(j0 == 2 * jj ? o.v0 : zero_h4, j0 == 2 * jj + 1 ? o.v0 : zero_h4),
-                                                            qf[jj], so, 0, 0, 0);
         }
-        const uint32_t r1 = o.fl & (o.fl - 1u);
-        if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
-            one(r1 ? __builtin_ctz(r1) : 255, o.v1);
-            uint32_t rem = r1 & (r1 - 1u);
-            int slot = o.slot + 2;
-            while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
-                const bool has = rem != 0;
-                one(has ? __builtin_ctz(rem) : 255, has ? outlier_chunk(p.Kc, DT, bh, slot) : zero_h4);
-                slot++;
-                rem &= rem - 1u;
-            }
+    };
+    auto k_apply = [&](const KPre &k, float4v (&so)[2]) {
+#pragma unroll
+        for (int bq = 0; bq < kKPre; bq++)
+            if (k.off[0] + 8 * bq < k.off[2]) k_batch(k.off, k.off[0] + 8 * bq, k.x[bq], k.cc[bq], so);
+        for (int bs = k.off[0] + 8 * kKPre; bs < k.off[2]; bs += 8) {      // more than the prefetched batches: rare
+            uint2 x[2];
+            uint32_t cc;
+            k_load(bs, x, cc);
+            k_batch(k.off, bs, x, cc, so);
         }
     };
     // V side: the verbatim chunks, transposed, times the unscaled probabilities of the tile.
@@ -486,20 +525,20 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.  A flagged chunk
     // carries radius code 0 in the main plane, so its decoded value is exactly zero and only the verbatim
     // value from the sideband contributes.
-    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const OutPre (&oc)[4]) {
-        float4v sT[2];
+    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre &kc, const OutPre (&oc)[2]) {
+        float4v sT[2], so[2] = {zero4, zero4};
+        if (FLAGS) k_apply(kc, so);
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
             decode_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, a);
-            float4v s = zero4, so = zero4;
+            float4v s = zero4;
 #pragma unroll
             for (int jj = 0; jj < CPL / 2; jj++)
                 s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
-            if (FLAGS) out_apply_k(oc[u], so);
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[e] * qmaxf : 0.f);
+                s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[u][e] * qmaxf : 0.f);
             sT[u] = s;
         }
         // ---- mask (boundary half-steps only), online softmax ----
@@ -552,49 +591,54 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
         }
         if (FLAGS) {
-            if (oc[2].any || oc[3].any) {   // the first flagged chunk of every lane, both tiles in one 16x16x32 MFMA
-                const int j0 = oc[2].fl ? __builtin_ctz(oc[2].fl) : 255, j1 = oc[3].fl ? __builtin_ctz(oc[3].fl) : 255;
+            if (oc[0].any || oc[1].any) {   // the first flagged chunk of every lane, both tiles in one 16x16x32 MFMA
+                const int j0 = oc[0].fl ? __builtin_ctz(oc[0].fl) : 255, j1 = oc[1].fl ? __builtin_ctz(oc[1].fl) : 255;
                 const half8 ppo = cat8(pTo[0], pTo[1]);
 #pragma unroll
                 for (int j = 0; j < CPL; j++) {
-                    const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(j0 == j ? oc[2].v0 : zero_h4, ident, zero4, 0, 0, 0);
-                    const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(j1 == j ? oc[3].v0 : zero_h4, ident, zero4, 0, 0, 0);
+                    const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(j0 == j ? oc[0].v0 : zero_h4, ident, zero4, 0, 0, 0);
+                    const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(j1 == j ? oc[1].v0 : zero_h4, ident, zero4, 0, 0, 0);
                     acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), ppo, acc[j], 0, 0, 0);
                 }
             }
-            out_apply_v(oc[2], pTo[0]);
-            out_apply_v(oc[3], pTo[1]);
+            out_apply_v(oc[0], pTo[0]);
+            out_apply_v(oc[1], pTo[1]);
         }
     };
 
-    // sideband requests of one half-step: K tiles 0, 1, then V tiles 0, 1
-    auto issue_all = [&](const FlagTile &f, OutPre (&o)[4]) {
-        out_issue(p.Kc, f.kfl[0], f.ksb[0], o[0]);
-        out_issue(p.Kc, f.kfl[1], f.ksb[1], o[1]);
-        out_issue(p.Vc, f.vfl[0], f.vsb[0], o[2]);
-        out_issue(p.Vc, f.vfl[1], f.vsb[1], o[3]);
+    // sideband requests of one half-step: the K batches, then V tiles 0, 1
+    auto issue_all = [&](const FlagTile &f, KPre &k, OutPre (&o)[2]) {
+        k_issue(f, k);
+        out_issue(v_side, v_cap1, f.vfl[0], f.vsb[0], o[0]);
+        out_issue(v_side, v_cap1, f.vfl[1], f.vsb[1], o[1]);
     };
-    OutPre oc[4] = {};
-    if (FLAGS && t_begin < t_end) issue_all(f0, oc);
+    OutPre oc[2] = {};
+    KPre kc = {};
+    if (FLAGS && t_begin < t_end) issue_all(f0, kc, oc);
 
     for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
         FastTile<NW, AB, FLAGS, NH> nxt;
         FlagTile f2 = {};
-        OutPre on[4] = {};
+        OutPre on[2] = {};
+        KPre kn = {};
         const bool more = t0 + STEP < t_end, more2 = t0 + 2 * STEP < t_end;
-        if (more) load_super(t0 + STEP, nxt);
         if (FLAGS) {
-            // flags two steps ahead, sideband chunks one step ahead (their flags were requested a step ago)
-            if (more2) load_flags(t0 + 2 * STEP, f2);
-            if (more) issue_all(f1, on);
+            // bookkeeping two steps ahead, sideband chunks one step ahead (their offsets were requested a step ago);
+            // past the end the current tile is requested again, see out_issue
+            load_super(more ? t0 + STEP : t0, nxt);
+            load_flags(more2 ? t0 + 2 * STEP : t0, f2);
+            issue_all(f1, kn, on);
+        } else if (more) {
+            load_super(t0 + STEP, nxt);
         }
-        half_step(cur.h[0], t0, oc);
-        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, oc);
+        half_step(cur.h[0], t0, kc, oc);
+        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, kc, oc);
         if (more) {
             cur = nxt;
             if (FLAGS) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) oc[i] = on[i];
+                for (int i = 0; i < 2; i++) oc[i] = on[i];
+                kc = kn;
                 f1 = f2;
             }
         }
@@ -645,7 +689,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
 template <int CPL, int MB, int AB, int IB, int DT>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
-    size_t shmem = (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    size_t shmem = flags ? (size_t)kQOffset + (size_t)CPL * 4 * 16 * 8 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 4) * sizeof(float);
     if (shmem < merge) shmem = merge;
     auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true> : attn_fast_kernel<CPL, MB, AB, IB, DT, false>;
@@ -680,6 +724,8 @@ int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, 
     // vector loads of plane rows: main rows 16-byte aligned (checked by the caller), aux and flag rows to their width
     if (p.aux_bits && (((uintptr_t)p.Kc.aux_plane | (uintptr_t)p.Vc.aux_plane) & 3)) return HQMQ_OK;
     if (flags && (((uintptr_t)p.Kc.flag_plane | (uintptr_t)p.Vc.flag_plane) & 3)) return HQMQ_OK;
+    if (flags && (!p.Kc.sb_coord || !p.Kc.sb_count || p.Kc.sb_cap < 2 || p.Vc.sb_cap < 2 || p.Kc.sb_cap >= (1 << 28) || p.Vc.sb_cap >= (1 << 28)))
+        return HQMQ_OK;     // the K side walks the entry list
     // 8-byte vector loads of Q rows, table rows and sideband chunks; strides were checked by the caller
     if (p.n == 32) {
         if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, st, handled);
