@@ -64,8 +64,7 @@ struct HalfTile {
 // chunks it points to can be requested a whole half-step before use
 struct FlagTile {
     int koff[3];               // K: sideband entries [koff[u], koff[u + 1]) belong to tile u (wave-uniform)
-    uint32_t vfl[2];           // V: flag bits of token `col` of tile u
-    int vsb[2];                // V: sideband slot of tile u's first flagged chunk
+    int voff[3];               // V: the same
 };
 // K outliers of one half-step, requested ahead: the first kKPre batches of eight sideband entries.  Lane
 // 16 * grp + col holds entries 2 * grp and 2 * grp + 1 of a batch (the same in all 16 lanes of a row).
@@ -74,6 +73,13 @@ struct KPre {
     int off[3];
     uint2 x[kKPre][2];         // verbatim chunks (raw bits of the cache dtype)
     uint32_t cc[kKPre];        // their coordinates: (token & 15) << 8 | chunk, two 16-bit fields
+};
+// V outliers of one half-step: the first NB batches of sixteen entries; lane 16 * grp + col holds entry `col`.
+template <int NB>
+struct VPre {
+    int off[3];
+    uint2 x[NB];
+    uint32_t cc[NB];
 };
 // the unit of prefetch: NH half-tiles (64 tokens; 32 for the variants with outlier flags, which need the registers)
 template <int NW, int AB, bool FLAGS, int NH>
@@ -113,6 +119,7 @@ __device__ __forceinline__ float scaled(float acc, uint32_t pair, int hi, float 
 // the V table at kVTabOffset, and a gather addresses them with idx * 8 (+ the instruction's immediate offset).
 constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
 constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chunk][column] fp16 chunks, after the V table
+constexpr int kSelOffset = kQOffset + 4096;        // outlier variants: nine rows of eight fp16, row r < 8 = unit vector r, row 8 = 0
 constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
@@ -293,15 +300,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const uint8_t *v_rows = p.Vc.main_plane + plane_row0 * mrb;
     const uint8_t *ka_rows = AB ? p.Kc.aux_plane + plane_row0 * arb : nullptr;
     const uint8_t *va_rows = AB ? p.Vc.aux_plane + plane_row0 * arb : nullptr;
-    const uint8_t *vf_rows = FLAGS ? p.Vc.flag_plane + plane_row0 * frb : nullptr;
     const int32_t *k_toff = FLAGS ? p.Kc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
     const int32_t *v_toff = FLAGS ? p.Vc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
     const uint32_t main_off = (uint32_t)(col * mrb + grp * NB), aux_off = (uint32_t)(col * arb + grp * ABYTES);
-    const uint32_t flag_off = (uint32_t)(col * frb), scale_off = (uint32_t)(4 * grp);
+    const uint32_t scale_off = (uint32_t)(4 * grp);
     const int k_count = FLAGS ? (int)min((int64_t)max(p.Kc.sb_count[bh], 0), p.Kc.sb_cap) : 0;
+    const int v_count = FLAGS ? (int)min((int64_t)max(p.Vc.sb_count[bh], 0), p.Vc.sb_cap) : 0;
     const char *k_side = FLAGS ? (const char *)p.Kc.sideband + (size_t)bh * p.Kc.sb_cap * 8 : nullptr;
     const char *v_side = FLAGS ? (const char *)p.Vc.sideband + (size_t)bh * p.Vc.sb_cap * 8 : nullptr;
     const char *k_coord = FLAGS ? (const char *)p.Kc.sb_coord + (size_t)bh * p.Kc.sb_cap * 2 : nullptr;
+    const char *v_coord = FLAGS ? (const char *)p.Vc.sb_coord + (size_t)bh * p.Vc.sb_cap * 2 : nullptr;
     const uint32_t k_cap1 = FLAGS ? (uint32_t)(p.Kc.sb_cap - 1) : 0u, v_cap1 = FLAGS ? (uint32_t)(p.Vc.sb_cap - 1) : 0u;
 
     auto load_super = [&](int t0, FastTile<NW, AB, FLAGS, NH> &s) {
@@ -338,16 +346,13 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         }
     }
     auto load_flags = [&](int th, FlagTile &f) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            f.vfl[u] = load_small<frb>(vf_rows + (size_t)th * frb + flag_off + u * 16 * frb);
-            f.vsb[u] = v_toff[(th >> 4) + u];
-        }
         // tiles not written yet hold INT32_MAX, and so does the slot after the last tile: the count bounds them
 #pragma unroll
         for (int i = 0; i < 3; i++) {
-            const int ti = (th >> 4) + i, v = k_toff[min(ti, tiles_cap1)];
-            f.koff[i] = min(ti <= tiles_cap1 ? v : 0x7fffffff, k_count);
+            const int ti = (th >> 4) + i, tc = min(ti, tiles_cap1);
+            const int kv = k_toff[tc], vv = v_toff[tc];
+            f.koff[i] = min(ti <= tiles_cap1 ? kv : 0x7fffffff, k_count);
+            f.voff[i] = min(ti <= tiles_cap1 ? vv : 0x7fffffff, v_count);
         }
     };
 
@@ -385,6 +390,10 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     if (max(Kk, Kv) > FU * NT)
         fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
+    if (FLAGS && threadIdx.x >= 64 && threadIdx.x < 100) {
+        const uint32_t w = threadIdx.x - 64, row = w >> 2, d = w & 3;
+        reinterpret_cast<uint32_t *>(lds_tab)[kSelOffset / 4 + w] = (row < 8 && (row >> 1) == d) ? 0x3C00u << (16 * (row & 1)) : 0u;
+    }
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
         for (int jj = 0; jj < CPL / 2; jj++) {
@@ -420,34 +429,8 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
     const half4 zero_h4 = half4{0, 0, 0, 0};
-    constexpr uint32_t cmask = (CPL >= 32) ? 0xffffffffu : ((1u << CPL) - 1u);
-    const int first = grp * CPL;
-
-    // Flag bookkeeping of one tile: the lane's CPL flag bits and the sideband slot of its first flagged chunk
-    // (tile offset + flagged chunks of earlier tokens of the tile + earlier chunks of the token).
-    auto lane_flags = [&](uint32_t fw, int tile_off, uint32_t &fl, int &slot) {
-        const int own = __popc(fw);
-        const int incl = row_prefix16(own);
-        fl = (fw >> first) & cmask;
-        slot = tile_off + incl - own + __popc(fw & ((1u << first) - 1u));
-    };
-
-    // Outlier chunks of one tile: flag bookkeeping done and the lane's first two sideband chunks requested.
-    struct OutPre {
-        bool any;           // some lane of the wavefront has a flagged chunk in this tile
-        uint32_t fl;        // the lane's CPL flag bits
-        int slot;           // sideband slot of its first flagged chunk
-        half4 v0, v1;       // its first two flagged chunks (requested early; more are rare and loaded on demand)
-    };
     // Every load of the loop is issued unconditionally (clamped addresses): a load inside a branch would make the
     // compiler's wait counts assume it was not issued, and the waits would then cover the next tile's prefetch.
-    auto out_issue = [&](const char *side, uint32_t cap1, uint32_t fw, int tile_off, OutPre &o) {
-        o.any = __builtin_amdgcn_ballot_w64(fw != 0) != 0;
-        lane_flags(fw, (int)min((uint32_t)tile_off, cap1), o.fl, o.slot);
-        const uint32_t s0 = min((uint32_t)o.slot, cap1), s1 = min((uint32_t)o.slot + 1u, cap1);
-        o.v0 = chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(side + s0 * 8u));
-        o.v1 = chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(side + s1 * 8u));
-    };
     // K side.  The sideband entries of a half-step are a contiguous range known from three tile offsets, so no
     // flag is read: a batch of eight entries is the reduction dimension of one MFMA per tile,
     //   so[token][column] += sum over entries e of the batch, i < 4:  [token(e) == token] x_e[i] * Q[column][4 chunk(e) + i],
@@ -495,37 +478,60 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             k_batch(k.off, bs, x, cc, so);
         }
     };
-    // V side: the verbatim chunks, transposed, times the unscaled probabilities of the tile.
-    auto out_apply_v = [&](const OutPre &o, half4 pTo) {      // second and further flagged chunks of a lane (rare)
-        if (!o.any) return;
-        auto one = [&](int jme, half4 val) {
+    // V side, also from the entry list, sixteen entries of the half-step per batch (lane 16 * grp + col holds
+    // entry `col`):
+    //   Pg[e][column] = P[token(e)][column]      one 16x16x32 MFMA: A = the unit vector of the entry's token slot
+    //                                            (LDS rows), B = the unscaled probabilities of the 32 tokens;
+    //   for every chunk position j in use:       X_j^T by the transposing MFMA (A = the entry's chunk in the row
+    //   acc[j] += X_j^T . Pg                     group that owns it, else zero), then one 16x16x16 MFMA over entries.
+    constexpr int kVPre = CPL >= 8 ? 2 : 1;
+    auto v_load = [&](int bs, uint2 &x, uint32_t &cc) {
+        const uint32_t e = min((uint32_t)bs + (uint32_t)col, v_cap1);
+        x = *reinterpret_cast<const uint2 *>(v_side + e * 8u);
+        cc = *reinterpret_cast<const uint16_t *>(v_coord + e * 2u);
+    };
+    auto v_issue = [&](const FlagTile &f, VPre<kVPre> &v) {
 #pragma unroll
-            for (int j = 0; j < CPL; j++) {
-                const bool mj = jme == j;
-                if (__builtin_amdgcn_ballot_w64(mj) != 0) {
-                    const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? val : zero_h4, ident, zero4, 0, 0, 0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pTo, acc[j], 0, 0, 0);
-                }
+        for (int i = 0; i < 3; i++) v.off[i] = f.voff[i];
+#pragma unroll
+        for (int bq = 0; bq < kVPre; bq++) v_load(v.off[0] + 16 * bq, v.x[bq], v.cc[bq]);
+    };
+    auto v_batch = [&](const int (&off)[3], int bs, uint2 x, uint32_t cc, half8 ppo) {
+        const int e = bs + col;
+        const bool ok = e < off[2];
+        const uint32_t ch = cc & (uint32_t)(n - 1), t = (cc >> 8) & 15u;
+        const uint32_t slot = (e >= off[1] ? 4u : 0u) + (t & 3u);             // position among the row group's 8 tokens
+        const bool mine = ok && (int)(t >> 2) == grp;
+        const uint4v sel = *(lds_u4_ptr)(uintptr_t)(kSelOffset + (mine ? slot : 8u) * 16u);
+        const half4 pg = pack4(__builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0));
+        const half4 h = chunk_to_half<DT>(x);
+        const bool owner = ok && (int)(ch / CPL) == grp;
+        const int jq = (int)(ch % CPL);
+#pragma unroll
+        for (int j = 0; j < CPL; j++) {
+            const bool mj = owner && jq == j;
+            if (__builtin_amdgcn_ballot_w64(mj) != 0) {
+                const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[j], 0, 0, 0);
             }
-        };
-        const uint32_t r1 = o.fl & (o.fl - 1u);
-        if (__builtin_amdgcn_ballot_w64(r1 != 0) != 0) {
-            one(r1 ? __builtin_ctz(r1) : 255, o.v1);
-            uint32_t rem = r1 & (r1 - 1u);
-            int slot = o.slot + 2;
-            while (__builtin_amdgcn_ballot_w64(rem != 0) != 0) {
-                const bool has = rem != 0;
-                one(has ? __builtin_ctz(rem) : 255, has ? outlier_chunk(p.Vc, DT, bh, slot) : zero_h4);
-                slot++;
-                rem &= rem - 1u;
-            }
+        }
+    };
+    auto v_apply = [&](const VPre<kVPre> &v, half8 ppo) {
+#pragma unroll
+        for (int bq = 0; bq < kVPre; bq++)
+            if (v.off[0] + 16 * bq < v.off[2]) v_batch(v.off, v.off[0] + 16 * bq, v.x[bq], v.cc[bq], ppo);
+        for (int bs = v.off[0] + 16 * kVPre; bs < v.off[2]; bs += 16) {     // more than the prefetched batches: rare
+            uint2 x;
+            uint32_t cc;
+            v_load(bs, x, cc);
+            v_batch(v.off, bs, x, cc, ppo);
         }
     };
 
     // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.  A flagged chunk
     // carries radius code 0 in the main plane, so its decoded value is exactly zero and only the verbatim
     // value from the sideband contributes.
-    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre &kc, const OutPre (&oc)[2]) {
+    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre &kc, const VPre<kVPre> &vc) {
         float4v sT[2], so[2] = {zero4, zero4};
         if (FLAGS) k_apply(kc, so);
 #pragma unroll
@@ -590,55 +596,40 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
         }
-        if (FLAGS) {
-            if (oc[0].any || oc[1].any) {   // the first flagged chunk of every lane, both tiles in one 16x16x32 MFMA
-                const int j0 = oc[0].fl ? __builtin_ctz(oc[0].fl) : 255, j1 = oc[1].fl ? __builtin_ctz(oc[1].fl) : 255;
-                const half8 ppo = cat8(pTo[0], pTo[1]);
-#pragma unroll
-                for (int j = 0; j < CPL; j++) {
-                    const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(j0 == j ? oc[0].v0 : zero_h4, ident, zero4, 0, 0, 0);
-                    const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(j1 == j ? oc[1].v0 : zero_h4, ident, zero4, 0, 0, 0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), ppo, acc[j], 0, 0, 0);
-                }
-            }
-            out_apply_v(oc[0], pTo[0]);
-            out_apply_v(oc[1], pTo[1]);
-        }
+        if (FLAGS) v_apply(vc, cat8(pTo[0], pTo[1]));
     };
 
-    // sideband requests of one half-step: the K batches, then V tiles 0, 1
-    auto issue_all = [&](const FlagTile &f, KPre &k, OutPre (&o)[2]) {
+    // sideband requests of one half-step
+    auto issue_all = [&](const FlagTile &f, KPre &k, VPre<kVPre> &v) {
         k_issue(f, k);
-        out_issue(v_side, v_cap1, f.vfl[0], f.vsb[0], o[0]);
-        out_issue(v_side, v_cap1, f.vfl[1], f.vsb[1], o[1]);
+        v_issue(f, v);
     };
-    OutPre oc[2] = {};
     KPre kc = {};
-    if (FLAGS && t_begin < t_end) issue_all(f0, kc, oc);
+    VPre<kVPre> vc = {};
+    if (FLAGS && t_begin < t_end) issue_all(f0, kc, vc);
 
     for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
         FastTile<NW, AB, FLAGS, NH> nxt;
         FlagTile f2 = {};
-        OutPre on[2] = {};
         KPre kn = {};
+        VPre<kVPre> vn = {};
         const bool more = t0 + STEP < t_end, more2 = t0 + 2 * STEP < t_end;
         if (FLAGS) {
-            // bookkeeping two steps ahead, sideband chunks one step ahead (their offsets were requested a step ago);
-            // past the end the current tile is requested again, see out_issue
+            // tile offsets two steps ahead, sideband entries one step ahead (their offsets were requested a step
+            // ago); past the end the current tile is requested again
             load_super(more ? t0 + STEP : t0, nxt);
             load_flags(more2 ? t0 + 2 * STEP : t0, f2);
-            issue_all(f1, kn, on);
+            issue_all(f1, kn, vn);
         } else if (more) {
             load_super(t0 + STEP, nxt);
         }
-        half_step(cur.h[0], t0, kc, oc);
-        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, kc, oc);
+        half_step(cur.h[0], t0, kc, vc);
+        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, kc, vc);
         if (more) {
             cur = nxt;
             if (FLAGS) {
-#pragma unroll
-                for (int i = 0; i < 2; i++) oc[i] = on[i];
                 kc = kn;
+                vc = vn;
                 f1 = f2;
             }
         }
@@ -689,7 +680,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
 template <int CPL, int MB, int AB, int IB, int DT>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
-    size_t shmem = flags ? (size_t)kQOffset + (size_t)CPL * 4 * 16 * 8 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 4) * sizeof(float);
     if (shmem < merge) shmem = merge;
     auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true> : attn_fast_kernel<CPL, MB, AB, IB, DT, false>;
@@ -723,8 +714,7 @@ int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, 
     if (p.t_cap % kSuper) return HQMQ_OK;
     // vector loads of plane rows: main rows 16-byte aligned (checked by the caller), aux and flag rows to their width
     if (p.aux_bits && (((uintptr_t)p.Kc.aux_plane | (uintptr_t)p.Vc.aux_plane) & 3)) return HQMQ_OK;
-    if (flags && (((uintptr_t)p.Kc.flag_plane | (uintptr_t)p.Vc.flag_plane) & 3)) return HQMQ_OK;
-    if (flags && (!p.Kc.sb_coord || !p.Kc.sb_count || p.Kc.sb_cap < 2 || p.Vc.sb_cap < 2 || p.Kc.sb_cap >= (1 << 28) || p.Vc.sb_cap >= (1 << 28)))
+    if (flags && (!p.Kc.sb_coord || !p.Kc.sb_count || !p.Vc.sb_coord || !p.Vc.sb_count || p.Kc.sb_cap < 2 || p.Vc.sb_cap < 2 || p.Kc.sb_cap >= (1 << 28) || p.Vc.sb_cap >= (1 << 28)))
         return HQMQ_OK;     // the K side walks the entry list
     // 8-byte vector loads of Q rows, table rows and sideband chunks; strides were checked by the caller
     if (p.n == 32) {

@@ -116,7 +116,9 @@ int hqmq_outlier_mask(const void *x, int64_t x_stride_b, int64_t x_stride_h, int
 
 /* Compact the flagged chunks of rows [row0, row0+T) into the sideband.
  * No counterpart in the reference (its wrapper keeps a dense tensor).
- * Rows must be appended in order; row0 = (pos ? pos[b] : 0) + t_off.
+ * Rows must be appended in order and each row once; row0 = (pos ? pos[b] : 0) + t_off.  (A row that is
+ * compacted a second time leaves its first entries in the list: the attention kernels that walk the list would
+ * count them twice.  To rewrite rows, reset sb_count and the tile offsets to the state before them.)
  * sb_coord [B][H][sb_cap] (may be NULL): (row & 15) << 8 | chunk of every sideband entry, which lets the
  * specialised attention kernels walk the sideband densely; sb_tile_off must start out as INT32_MAX (tiles not
  * yet written read as "no entries"). */
