@@ -109,6 +109,8 @@ def run(cfg, steps):
     cache.K.check_overflow()
     cache.V.check_overflow()
     lens_dev = lens.to(DEV) if lens is not None else None
+    if lens is not None:
+        cache.crop_(lens_dev)                    # every sequence keeps its own context; the rows behind it are free
     Q = torch.randn(B, Hq, 1, d, generator=torch.Generator(device=DEV).manual_seed(7), device=DEV).to(dt)
     out = torch.empty_like(Q)
     err, ref_max = dense_check(Q, cache, lens, T)

@@ -152,13 +152,16 @@ __device__ __forceinline__ void tile_flags(const PackedDev &c, size_t plane_row0
     const uint32_t fw_t = (uint32_t)__shfl((int)fw, tok, 16);
     const int pre_t = __shfl(pre, tok, 16);
     fl = (fw_t >> first) & ((CPL >= 32) ? 0xffffffffu : ((1u << CPL) - 1u));
-    slot0 = c.sb_tile_off[tile_off_index] + pre_t + __popc(fw_t & ((first >= 32) ? 0xffffffffu : ((1u << first) - 1u)));
+    // tiles never written (or cropped) hold INT32_MAX: bound the offset before adding to it
+    const int tile_off = min(c.sb_tile_off[tile_off_index], (int)min(c.sb_cap, (int64_t)0x3fffffff));
+    slot0 = max(tile_off, 0) + pre_t + __popc(fw_t & ((first >= 32) ? 0xffffffffu : ((1u << first) - 1u)));
 }
 
 // A flagged chunk: the verbatim values from the sideband (exact in fp16 for fp16 caches).
 __device__ __forceinline__ half4 outlier_chunk(const PackedDev &c, int dtype, size_t bh, int slot) {
     int64_t s = slot;
     if (s >= c.sb_cap) s = c.sb_cap - 1;
+    if (s < 0) s = 0;
     return load_chunk_h(c.sideband, dtype, (int64_t)bh * c.sb_cap + s);
 }
 

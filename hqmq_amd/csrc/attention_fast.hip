@@ -354,6 +354,12 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             f.koff[i] = min(ti <= tiles_cap1 ? kv : 0x7fffffff, k_count);
             f.voff[i] = min(ti <= tiles_cap1 ? vv : 0x7fffffff, v_count);
         }
+        // a tile has at most 16 n entries: bounds the walk if the caller's offsets are inconsistent
+#pragma unroll
+        for (int i = 1; i < 3; i++) {
+            f.koff[i] = min(f.koff[i], f.koff[i - 1] + 16 * n);
+            f.voff[i] = min(f.voff[i], f.voff[i - 1] + 16 * n);
+        }
     };
 
     // First batch of codeword-table loads (the longest dependency chain of the prologue: load, convert, LDS

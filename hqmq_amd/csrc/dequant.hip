@@ -108,11 +108,13 @@ __global__ void dequant_packed_kernel(PackedView p, int B, int H, int T, int n, 
         ST *dst = out + g * 4;
         if (p.flag_plane && ((p.flag_plane[prow * frb + (c >> 3)] >> (c & 7)) & 1)) {
             const int tile = t >> 4;
-            int rank = p.sb_tile_off[bh * ((t_cap + kTile - 1) / kTile) + tile];
+            // 64-bit and clamped on both sides: a tile that was never written (or was cropped) holds INT32_MAX
+            int64_t rank = p.sb_tile_off[bh * ((t_cap + kTile - 1) / kTile) + tile];
             for (int tt = tile * kTile; tt < t; tt++)
                 for (int by = 0; by < frb; by++) rank += __popc((uint32_t)p.flag_plane[(bh * t_cap + tt) * frb + by]);
             for (int cc = 0; cc < c; cc++) rank += (p.flag_plane[prow * frb + (cc >> 3)] >> (cc & 7)) & 1;
-            const ST *src = (const ST *)p.sideband + (bh * p.sb_cap + (rank < p.sb_cap ? rank : p.sb_cap - 1)) * 4;
+            rank = rank < 0 ? 0 : (rank < p.sb_cap ? rank : p.sb_cap - 1);
+            const ST *src = (const ST *)p.sideband + (bh * p.sb_cap + rank) * 4;
             for (int j = 0; j < 4; j++) dst[j] = src[j];
             continue;
         }

@@ -15,7 +15,7 @@ PackedQuantizedCache  +  attn_implementation="hqmq_packed"
     out = model(input_ids, past_key_values=cache, use_cache=True)
 
 Limits: unpadded batches (every sequence of the batch has the same length; the causal mask is the only mask),
-no cache cropping / beam reordering.  This module imports `transformers`; nothing else in the package does.
+no beam reordering (cropping is supported).  This module imports `transformers`; nothing else in the package does.
 """
 from __future__ import annotations
 
@@ -75,8 +75,16 @@ class PackedLayer(DynamicLayer):
     def get_max_length(self) -> int:
         return self.max_tokens
 
-    def crop(self, *args, **kwargs):
-        raise NotImplementedError("a packed cache cannot be cropped")
+    def crop(self, tokens_to_remove: int) -> None:
+        """Drops the last -tokens_to_remove tokens (DynamicLayer.crop; a positive value is its older meaning: the
+        length to keep)."""
+        if self.packed is None or tokens_to_remove == 0:
+            return
+        keep = tokens_to_remove if tokens_to_remove > 0 else max(self.n_tokens + tokens_to_remove, 0)
+        if keep >= self.n_tokens:
+            return
+        self.packed.crop_(keep)
+        self.n_tokens = keep
 
     def batch_repeat_interleave(self, repeats: int) -> None:
         raise NotImplementedError("a packed cache cannot be repeated along the batch")

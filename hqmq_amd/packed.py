@@ -89,6 +89,37 @@ class PackedTensor:
         s.joint, s.joint_sh, s.K = L.ptr(self.joint), self.joint.stride(0), self.joint.shape[1]
         return s
 
+    def crop_(self, lengths) -> None:
+        """Forgets the rows from `lengths` on (an int for all sequences or an int tensor [B]): the outlier list and
+        its tile offsets go back to the state after the last kept row, so that the rows can be appended again.
+        The planes themselves are left as they are (later appends overwrite them)."""
+        B, H = self.B, self.H
+        if isinstance(lengths, int):
+            lens = torch.full((B,), lengths, dtype=torch.int64, device=self.device)
+            self.length = min(self.length, lengths)
+        else:
+            lens = lengths.to(device=self.device, dtype=torch.int64).clamp(min=0)
+            self.lengths = lens.to(torch.int32)
+        if self.flags is None:
+            return
+        tiles = self.t_cap // TILE
+        tile, r = lens // TILE, lens % TILE
+        tc = tile.clamp(max=tiles - 1)
+        off = self.sb_tile_off.gather(2, tc.view(B, 1, 1).expand(B, H, 1)).squeeze(2).to(torch.int64)
+        # flagged chunks of the kept rows of the tile the cut falls into
+        rows = tc.view(B, 1, 1) * TILE + torch.arange(TILE, device=self.device).view(1, 1, TILE)
+        fl = self.flags.gather(2, rows.view(B, 1, TILE, 1).expand(B, H, TILE, self.flags.shape[-1]))
+        bits = sum((fl >> i) & 1 for i in range(8)).to(torch.int64).sum(-1)                          # (B, H, TILE)
+        kept = torch.arange(TILE, device=self.device).view(1, 1, TILE) < r.view(B, 1, 1)
+        count = self.sb_count.to(torch.int64)
+        new = torch.where((tile >= tiles).view(B, 1) | (off > count), count, off + (bits * kept).sum(-1))
+        self.sb_count.copy_(torch.minimum(new, count).to(torch.int32))
+        first_free = (lens + TILE - 1) // TILE             # tiles from here on hold no kept row: unwritten again
+        gone = torch.arange(tiles, device=self.device).view(1, 1, tiles) >= first_free.view(B, 1, 1)
+        self.sb_tile_off.masked_fill_(gone.expand(B, H, tiles), 0x7fffffff)
+        dropped = torch.arange(self.t_cap, device=self.device).view(1, 1, self.t_cap, 1) >= lens.view(B, 1, 1, 1)
+        self.flags.masked_fill_(dropped, 0)                # no flag without an entry behind it
+
     def check_overflow(self) -> None:
         """Raises if an append ran out of sideband room (reads one int from the device)."""
         if self.sb_overflow is not None and int(self.sb_overflow.item()):
@@ -108,3 +139,8 @@ class PackedKV:
 
     def nbytes(self, length: Optional[int] = None) -> int:
         return self.K.nbytes(length) + self.V.nbytes(length)
+
+    def crop_(self, lengths) -> None:
+        """Forgets the rows from `lengths` on in K and V (see PackedTensor.crop_)."""
+        self.K.crop_(lengths)
+        self.V.crop_(lengths)

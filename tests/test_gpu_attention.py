@@ -306,3 +306,81 @@ def test_clustered_outlier_channels(d_h, Tq, hot, dn):
         for ns in (0, 3):
             O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, force_generic=generic, n_splits=ns)
             assert (O.float() - ref).abs().max().item() < tol, (generic, ns)
+
+
+def _planted(B, H, T, d, seed, dt):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, H, T, d, generator=g)
+    hit = torch.rand(B, H, T, d // 4, 1, generator=g) < 0.04
+    x = torch.where(hit, x.view(B, H, T, d // 4, 4) * 40.0, x.view(B, H, T, d // 4, 4)).reshape(B, H, T, d)
+    return x.to(dt).to(DEV)
+
+
+def test_crop_then_append_again_equals_never_appended():
+    """crop_ puts the outlier list and its tile offsets back to the state after the last kept row: rows appended,
+    cropped and appended again give the same planes, the same list and the same attention output as a cache that
+    never saw the cropped rows (same calls otherwise, so the per-call medians agree)."""
+    import hqmq
+    dt = torch.float16
+    B, Hq, Hkv, T, d_h = 2, 8, 2, 200, 128
+    k, v = _planted(B, Hkv, T, d_h, 11, dt), _planted(B, Hkv, T, d_h, 12, dt)
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    a = w.new_cache(B, T + 40, d_h, dt, 0, sideband_frac=0.5)
+    w.append(a, k[:, :, :150], v[:, :, :150], 0)
+    w.append(a, k[:, :, 150:], v[:, :, 150:], 0)
+    b = w.new_cache(B, T + 40, d_h, dt, 0, sideband_frac=0.5)
+    w.append(b, k[:, :, :150], v[:, :, :150], 0)
+    w.append(b, k[:, :, 40:75], v[:, :, 40:75], 0)          # 35 rows that are dropped again (the cut is inside a tile)
+    b.crop_(150)
+    assert b.length == 150
+    w.append(b, k[:, :, 150:], v[:, :, 150:], 0)
+    for pa, pb in ((a.K, b.K), (a.V, b.V)):
+        assert int(pa.sb_count.min()) > 0 and torch.equal(pa.sb_count, pb.sb_count)
+        assert torch.equal(pa.sb_tile_off, pb.sb_tile_off)
+        for x, y in ((pa.main, pb.main), (pa.flags, pb.flags), (pa.scale.view(torch.int16), pb.scale.view(torch.int16))):
+            assert torch.equal(x[:, :, :T], y[:, :, :T])
+        for bb in range(B):
+            for h in range(Hkv):
+                c = int(pa.sb_count[bb, h])
+                assert torch.equal(pa.sideband[bb, h, :c].view(torch.int16), pb.sideband[bb, h, :c].view(torch.int16))
+                assert torch.equal(pa.sb_coord[bb, h, :c], pb.sb_coord[bb, h, :c])
+    Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(13)).to(dt).to(DEV)
+    Oa = hqmq.fused_attention_packed(Q, a, causal=False)
+    for generic in (False, True):
+        assert torch.equal(hqmq.fused_attention_packed(Q, b, causal=False, force_generic=generic),
+                           Oa if not generic else hqmq.fused_attention_packed(Q, a, causal=False, force_generic=True))
+
+
+def test_crop_per_sequence_then_decode_appends():
+    """Ragged crop (tile-aligned and not), then appends at pos: specialised and layout-generic kernels against dense
+    attention over the dequantized cache with per-sequence lengths."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.bfloat16
+    B, Hq, Hkv, T, d_h = 3, 8, 2, 160, 64
+    k, v = _planted(B, Hkv, T, d_h, 21, dt), _planted(B, Hkv, T, d_h, 22, dt)
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    cache = w.new_cache(B, T + 64, d_h, dt, 0, sideband_frac=0.5)
+    w.append(cache, k, v, 0)
+    lens = torch.tensor([150, 128, 37], dtype=torch.int32, device=DEV)
+    cache.crop_(lens)
+    pos = lens.clone()
+    for step in range(20):                                   # crosses tile boundaries in every sequence
+        w.append(cache, k[:, :, step:step + 1], v[:, :, step:step + 1], 0, pos=pos)
+        pos += 1
+    cache.K.check_overflow()
+    Tm = int(pos.max())
+    Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(23)).to(dt).to(DEV)
+    Kd = ops.dequant_packed(cache.K, Tm, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, Tm, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    mask = torch.arange(Tm, device=DEV).view(1, 1, 1, Tm) < pos.view(B, 1, 1, 1)
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
+    # the appended rows really are the new tokens: row lens[b] + i decodes to (about) k[b, :, i]
+    for bb in range(B):
+        got = ops.dequant_packed(cache.K, Tm, 0)[bb, :, int(lens[bb]):int(lens[bb]) + 20].float()
+        assert (got - k[bb, :, :20].float()).abs().mean().item() < 0.25 * k[bb, :, :20].float().abs().mean().item()
+    tol = 8e-3 * max(1.0, float(ref.abs().max()))
+    for generic in (False, True):
+        O = hqmq.fused_attention_packed(Q, cache, causal=False, kv_lens=pos, T_kv=Tm, force_generic=generic)
+        assert (O.float() - ref).abs().max().item() < tol, generic

@@ -64,3 +64,35 @@ def test_packed_cache_matches_fake_quant_cache(dn, med3x):
     # compressed size: 4 bits/value of codes + the per-token scale (+ flags and sideband with Med3x)
     dense_bytes = 3 * 2 * 2 * 2 * ids.shape[1] * 64 * 2
     assert packed.nbytes() < (0.6 if med3x else 0.36) * dense_bytes
+
+
+def test_packed_cache_crop_replays_identically():
+    """Rolling the packed cache back (speculative decoding) and decoding the same tokens again gives the same logits
+    bit for bit, with outliers on both sides of the cut."""
+    import hqmq
+    from src.model_utils import ATTN_NAME, PackedQuantizedCache
+    model = tiny_llama(torch.float16)
+    q = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=3, n_heads=2, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    with torch.no_grad():
+        for layer in model.model.layers:
+            layer.self_attn.k_proj.weight[8:16] *= 12.0
+            layer.self_attn.v_proj.weight[40:44] *= 12.0
+    ids = torch.randint(0, 256, (2, 150), generator=torch.Generator().manual_seed(2)).to(DEV)
+    model.set_attn_implementation(ATTN_NAME)
+    cache = PackedQuantizedCache(q, max_tokens=256, sideband_frac=0.5)
+
+    def decode(first, last):
+        with torch.no_grad():
+            return torch.stack([model(ids[:, t:t + 1], past_key_values=cache, use_cache=True).logits[:, -1].float()
+                                for t in range(first, last)])
+    with torch.no_grad():
+        model(ids[:, :139], past_key_values=cache, use_cache=True)
+    once = decode(139, 146)
+    counts = [int(layer.packed.K.sb_count.sum()) for layer in cache.layers]
+    cache.crop(-5)
+    assert cache.get_seq_length() == 141
+    assert all(int(layer.packed.K.sb_count.sum()) < c for layer, c in zip(cache.layers, counts))
+    again = decode(141, 146)
+    cache.check_overflow()
+    assert cache.get_seq_length() == 146 and torch.equal(once[2:], again)
+    assert [int(layer.packed.K.sb_count.sum()) for layer in cache.layers] == counts
