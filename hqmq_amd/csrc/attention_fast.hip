@@ -81,7 +81,7 @@ struct VPre {
     uint2 x[NB];
     uint32_t cc[NB];
 };
-// the unit of prefetch: NH half-tiles (64 tokens; 32 for the variants with outlier flags, which need the registers)
+// the unit of prefetch: NH half-tiles of 32 tokens
 template <int NW, int AB, bool FLAGS, int NH>
 struct FastTile {
     HalfTile<NW, AB, FLAGS> h[NH];
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = kFastWaves * 64;
-    constexpr int NH = FLAGS ? 1 : 2, STEP = 32 * NH;
+    constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
 
