@@ -29,7 +29,7 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the attention kernel from the FETCH_SIZE / WRITE_SIZE passes (scaled by a plain
 # 256 MiB copy), recorded in profiles/attn_fast_kernel_config2_32k_hbm_traffic.txt; known for these contexts only.
-MEASURED_TRAFFIC_BYTES = {32768: 37.80e6}
+MEASURED_TRAFFIC_BYTES = {32768: 37.73e6}
 
 
 def build_cache(q, T, dt, dev, seed):

@@ -646,14 +646,14 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const float l_tot = row_sum4(l_run);
     float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][RS]
     __syncthreads();
-    {
+    const int ncols = min(16, p.Tq * G - cg * 16);
+    if (col < ncols) {                                          // padding columns are never read back
         float *wp = red + ((size_t)wave * 16 + col) * RS;
         if (grp == 0) { wp[d_h] = m_run; wp[d_h + 1] = l_tot; }
 #pragma unroll
         for (int j = 0; j < CPL; j++) *reinterpret_cast<float4v *>(wp + grp * CPL * 4 + 4 * j) = acc[j];
     }
     __syncthreads();
-    const int ncols = min(16, p.Tq * G - cg * 16);
     const float inv_qmax = p.inv_qmax;
     for (int o = threadIdx.x; o < ncols * d_h; o += NT) {
         const int cc = o / d_h, e = o - cc * d_h;
