@@ -66,13 +66,13 @@ struct FlagTile {
     int koff[3];               // K: sideband entries [koff[u], koff[u + 1]) belong to tile u (wave-uniform)
     int voff[3];               // V: the same
 };
-// K outliers of one half-step, requested ahead: the first kKPre batches of eight sideband entries.  Lane
+// K outliers of one half-step, requested ahead: the first NB batches of eight sideband entries.  Lane
 // 16 * grp + col holds entries 2 * grp and 2 * grp + 1 of a batch (the same in all 16 lanes of a row).
-constexpr int kKPre = 2;
+template <int NB>
 struct KPre {
     int off[3];
-    uint2 x[kKPre][2];         // verbatim chunks (raw bits of the cache dtype)
-    uint32_t cc[kKPre];        // their coordinates: (token & 15) << 8 | chunk, two 16-bit fields
+    uint2 x[NB][2];            // verbatim chunks (raw bits of the cache dtype)
+    uint32_t cc[NB];           // their coordinates: (token & 15) << 8 | chunk, two 16-bit fields
 };
 // V outliers of one half-step: the first NB batches of sixteen entries; lane 16 * grp + col holds entry `col`.
 template <int NB>
@@ -253,6 +253,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = kFastWaves * 64;
+    constexpr int kKPre = CPL >= 8 ? 2 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
@@ -448,7 +449,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         x[1] = *reinterpret_cast<const uint2 *>(k_side + e1 * 8u);
         cc = (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e0 * 2u) | (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e1 * 2u) << 16;
     };
-    auto k_issue = [&](const FlagTile &f, KPre &k) {
+    auto k_issue = [&](const FlagTile &f, KPre<kKPre> &k) {
 #pragma unroll
         for (int i = 0; i < 3; i++) k.off[i] = f.koff[i];
 #pragma unroll
@@ -473,7 +474,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             }
         }
     };
-    auto k_apply = [&](const KPre &k, float4v (&so)[2]) {
+    auto k_apply = [&](const KPre<kKPre> &k, float4v (&so)[2]) {
 #pragma unroll
         for (int bq = 0; bq < kKPre; bq++)
             if (k.off[0] + 8 * bq < k.off[2]) k_batch(k.off, k.off[0] + 8 * bq, k.x[bq], k.cc[bq], so);
@@ -537,7 +538,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     // One half-step: 32 tokens (two tiles) through scores, online softmax and the V product.  A flagged chunk
     // carries radius code 0 in the main plane, so its decoded value is exactly zero and only the verbatim
     // value from the sideband contributes.
-    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre &kc, const VPre<kVPre> &vc) {
+    auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre<kKPre> &kc, const VPre<kVPre> &vc) {
         float4v sT[2], so[2] = {zero4, zero4};
         if (FLAGS) k_apply(kc, so);
 #pragma unroll
@@ -606,18 +607,18 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     };
 
     // sideband requests of one half-step
-    auto issue_all = [&](const FlagTile &f, KPre &k, VPre<kVPre> &v) {
+    auto issue_all = [&](const FlagTile &f, KPre<kKPre> &k, VPre<kVPre> &v) {
         k_issue(f, k);
         v_issue(f, v);
     };
-    KPre kc = {};
+    KPre<kKPre> kc = {};
     VPre<kVPre> vc = {};
     if (FLAGS && t_begin < t_end) issue_all(f0, kc, vc);
 
     for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
         FastTile<NW, AB, FLAGS, NH> nxt;
         FlagTile f2 = {};
-        KPre kn = {};
+        KPre<kKPre> kn = {};
         VPre<kVPre> vn = {};
         const bool more = t0 + STEP < t_end, more2 = t0 + 2 * STEP < t_end;
         if (FLAGS) {

@@ -213,6 +213,101 @@ __global__ __launch_bounds__(1024) void med_select1_kernel(uint32_t *ws, int H, 
     }
 }
 
+// Small calls (a decode step appends B * n chunks per head): norms, exact radix select and count in one launch,
+// one block per head, the 16-bit keys in LDS.  16-bit dtypes only.
+constexpr int kSmallMax = 8192;
+
+// rank -> (bin holding it, rank inside the bin) over the 256 counters of `hist`; every thread of the block calls it
+__device__ __forceinline__ void find_bin256(const uint32_t *hist, uint32_t rank, uint32_t *wave_tot, uint32_t *res,
+                                            uint32_t &bin, uint32_t &inner) {
+    const int tid = threadIdx.x;
+    uint32_t v = 0, incl = 0;
+    if (tid < 256) {
+        v = hist[tid];
+        incl = v;
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t u = __shfl_up(incl, o, 64);
+            if ((tid & 63) >= o) incl += u;
+        }
+        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        for (int w = 0; w < (tid >> 6); w++) incl += wave_tot[w];
+        const uint32_t excl = incl - v;
+        if (rank >= excl && rank < incl) { res[0] = (uint32_t)tid; res[1] = rank - excl; }
+    }
+    __syncthreads();
+    bin = res[0];
+    inner = res[1];
+    __syncthreads();
+}
+
+template <class D>
+__global__ __launch_bounds__(1024) void med_small_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int B,
+                                                         int T, int n, float mult, float *median, typename D::storage *thr,
+                                                         int32_t *n_out) {
+    __shared__ uint16_t keys[kSmallMax];
+    __shared__ uint32_t hist[256], wave_tot[4], res[2], nan_count, gt_count;
+    __shared__ float thr_sh;
+    const int h = blockIdx.x, tid = threadIdx.x;
+    const int per_head = B * T * n;
+    if (tid == 0) { nan_count = 0; gt_count = 0; res[0] = 255; res[1] = 0; }
+    __syncthreads();
+    for (int g = tid; g < per_head; g += 1024) {
+        const int bt = g / n, c = g - bt * n, b = bt / T, t = bt - b * T;
+        const float nrm = chunk_norm<D>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4);
+        if (is_nan(nrm)) { atomicAdd(&nan_count, 1u); keys[g] = 0xffffu; }
+        else keys[g] = (uint16_t)(norm_bits<D>(nrm) >> 16);
+    }
+    __syncthreads();
+    if (nan_count > 0) {  // a NaN norm makes the quantile NaN, the mask empty
+        if (tid == 0) {
+            median[h] = NAN;
+            D::store(thr + h, NAN);
+            if (n_out) n_out[h] = 0;
+        }
+        return;
+    }
+    auto select = [&](uint32_t rank) -> uint32_t {
+        uint32_t hi, in_hi, lo, in_lo;
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        for (int g = tid; g < per_head; g += 1024) atomicAdd(&hist[keys[g] >> 8], 1u);
+        __syncthreads();
+        find_bin256(hist, rank, wave_tot, res, hi, in_hi);
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        for (int g = tid; g < per_head; g += 1024)
+            if ((uint32_t)(keys[g] >> 8) == hi) atomicAdd(&hist[keys[g] & 255u], 1u);
+        __syncthreads();
+        find_bin256(hist, in_hi, wave_tot, res, lo, in_lo);
+        return (hi << 8) | lo;
+    };
+    const uint32_t r_lo = (uint32_t)((per_head - 1) / 2), r_hi = (uint32_t)(per_head / 2);
+    const uint32_t klo = select(r_lo);
+    const uint32_t khi = r_hi == r_lo ? klo : select(r_hi);
+    if (tid == 0) {
+        const float a = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)klo)) : __uint_as_float(klo << 16);
+        const float b = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)khi)) : __uint_as_float(khi << 16);
+        finish_threshold<D>(a, b, r_lo == r_hi, mult, h, median, thr);
+        thr_sh = D::load(thr + h);
+    }
+    __syncthreads();
+    if (n_out) {
+        const float tv = thr_sh;
+        uint32_t cnt = 0;
+        for (int g = tid; g < per_head; g += 1024) {
+            const uint32_t k = keys[g];
+            const float v = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)k)) : __uint_as_float(k << 16);
+            if (v > tv) cnt++;
+        }
+        if (cnt) atomicAdd(&gt_count, cnt);
+        __syncthreads();
+        if (tid == 0) n_out[h] = (int32_t)gt_count;
+    }
+}
+
 __global__ __launch_bounds__(1024) void med_select2_kernel(uint32_t *ws, int H, int64_t per_head, float mult, float *median,
                                                            float *thr) {
     const int h = blockIdx.x;
@@ -393,8 +488,13 @@ static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B
     using ST = typename D::storage;
     const bool f32 = D::code == HQMQ_F32;
     const int64_t words = ws_words(H, f32);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, ws, words);
     const int64_t per_head = (int64_t)B * T * n;
+    if (!f32 && per_head <= kSmallMax) {
+        hipLaunchKernelGGL(med_small_kernel<D>, dim3(H), dim3(1024), 0, st, (const ST *)x, xsb, xsh, xst, B, T, n, mult, median,
+                           (ST *)thr, n_out);
+        return hip_status(hipGetLastError());
+    }
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, ws, words);
     int gx = (int)((per_head + 255) / 256);
     if (gx > 2048) gx = 2048;
     if (per_head >= (1 << 18)) {
