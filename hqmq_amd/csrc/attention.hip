@@ -345,24 +345,24 @@ static PackedDev to_dev(const hqmq_packed &k) {
 }
 
 template <int CPL, int MB>
-static int launch_attn(const AttnParams &p, bool flags, dim3 grid, size_t shmem, hipStream_t st) {
+static int launch_attn(const AttnParams &p, bool flags, dim3 grid, size_t shmem, hipStream_t st, const LaunchTiming &tm) {
     auto kern = flags ? attn_kernel<CPL, MB, true> : attn_kernel<CPL, MB, false>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(kAttnWaves * 64), shmem, st, p);
+    launch_timed(kern, grid, dim3(kAttnWaves * 64), shmem, st, tm, p);
     return hip_status(hipGetLastError());
 }
 
 template <int CPL>
-static int launch_attn_mb(const AttnParams &p, int mb, bool flags, dim3 grid, size_t shmem, hipStream_t st) {
+static int launch_attn_mb(const AttnParams &p, int mb, bool flags, dim3 grid, size_t shmem, hipStream_t st, const LaunchTiming &tm) {
     switch (mb) {
-        case 8: return launch_attn<CPL, 8>(p, flags, grid, shmem, st);
+        case 8: return launch_attn<CPL, 8>(p, flags, grid, shmem, st, tm);
         case 12:
-            if constexpr (CPL % 2 == 0) return launch_attn<CPL, 12>(p, flags, grid, shmem, st);
+            if constexpr (CPL % 2 == 0) return launch_attn<CPL, 12>(p, flags, grid, shmem, st, tm);
             else return HQMQ_ERR_SHAPE;
-        case 16: return launch_attn<CPL, 16>(p, flags, grid, shmem, st);
+        case 16: return launch_attn<CPL, 16>(p, flags, grid, shmem, st, tm);
         default: return HQMQ_ERR_LAYOUT;
     }
 }
@@ -470,20 +470,23 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     if (p.n_cg > 65535) return HQMQ_ERR_SHAPE;
     dim3 grid((unsigned)n_splits, (unsigned)p.n_cg, (unsigned)(a->B * a->H_kv));
     hipStream_t st = (hipStream_t)stream;
+    LaunchTiming tm;
+    tm.start = (hipEvent_t)a->start_event;
+    tm.stop = (hipEvent_t)a->stop_event;
     int rc = HQMQ_OK;
     bool handled = false;
     if (p.scale_vec && !a->force_generic && a->softmax_scale > 0.f) {
-        rc = launch_attn_fast(p, a->main_bits, flags, grid, ((size_t)a->K.K + a->V.K) * 8, st, &handled);
+        rc = launch_attn_fast(p, a->main_bits, flags, grid, ((size_t)a->K.K + a->V.K) * 8, st, tm, &handled);
         if (rc) return rc;
     }
     if (!handled) switch (n / 4) {
-        case 1: rc = launch_attn_mb<1>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 2: rc = launch_attn_mb<2>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 4: rc = launch_attn_mb<4>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 5: rc = launch_attn_mb<5>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 8: rc = launch_attn_mb<8>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 10: rc = launch_attn_mb<10>(p, a->main_bits, flags, grid, shmem, st); break;
-        case 16: rc = launch_attn_mb<16>(p, a->main_bits, flags, grid, shmem, st); break;
+        case 1: rc = launch_attn_mb<1>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 2: rc = launch_attn_mb<2>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 4: rc = launch_attn_mb<4>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 5: rc = launch_attn_mb<5>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 8: rc = launch_attn_mb<8>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 10: rc = launch_attn_mb<10>(p, a->main_bits, flags, grid, shmem, st, tm); break;
+        case 16: rc = launch_attn_mb<16>(p, a->main_bits, flags, grid, shmem, st, tm); break;
         default: return HQMQ_ERR_SHAPE;
     }
     if (rc) return rc;

@@ -1,6 +1,7 @@
 // Types and device helpers shared by the generic and the specialised attention kernels.
 #pragma once
 #include "common.h"
+#include <hip/hip_ext.h>
 
 namespace hqmq {
 
@@ -189,6 +190,17 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
 // Implemented in attention_fast.hip: kernels specialised at compile time for the common layouts
 // (d_h 64/128, fp16/bf16 caches, 16+0 / 12+1 / 16+3 bit codes). Returns HQMQ_OK and sets *handled when
 // it launched one of them; otherwise the caller falls back to the generic kernel.
-int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled);
+// Optional events that receive the GPU timestamps of the begin and the end of the main attention kernel.
+struct LaunchTiming {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+template <class Kern>
+inline void launch_timed(Kern kern, dim3 grid, dim3 block, size_t shmem, hipStream_t st, const LaunchTiming &tm, const AttnParams &p) {
+    if (tm.start || tm.stop) hipExtLaunchKernelGGL(kern, grid, block, shmem, st, tm.start, tm.stop, 0, p);
+    else hipLaunchKernelGGL(kern, grid, block, shmem, st, p);
+}
+
+int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st,
+                     const LaunchTiming &tm, bool *handled);
 
 }  // namespace hqmq

@@ -685,7 +685,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
 }
 
 template <int CPL, int MB, int AB, int IB, int DT>
-static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st) {
+static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
     size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 4) * sizeof(float);
@@ -695,25 +695,26 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(kFastWaves * 64), shmem, st, p);
+    launch_timed(kern, grid, dim3(kFastWaves * 64), shmem, st, tm, p);
     return hip_status(hipGetLastError());
 }
 
 template <int CPL, int DT>
-static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, bool *handled) {
+static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
     *handled = true;
-    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st);
-    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st);
-    if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st);
-    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st);
+    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
+    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st, tm);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st, tm);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st, tm);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st, tm);
     *handled = false;
     return HQMQ_OK;
 }
 
-int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st, bool *handled) {
+int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st,
+                     const LaunchTiming &tm, bool *handled) {
     (void)table_bytes;
     *handled = false;
     if (p.dtype != HQMQ_F16 && p.dtype != HQMQ_BF16) return HQMQ_OK;
@@ -725,11 +726,11 @@ int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, 
         return HQMQ_OK;     // the K side walks the entry list
     // 8-byte vector loads of Q rows, table rows and sideband chunks; strides were checked by the caller
     if (p.n == 32) {
-        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, st, handled);
-        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, st, handled);
+        if (p.dtype == HQMQ_F16) return launch_layout<8, HQMQ_F16>(p, main_bits, flags, grid, st, tm, handled);
+        return launch_layout<8, HQMQ_BF16>(p, main_bits, flags, grid, st, tm, handled);
     }
-    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, st, handled);
-    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, st, handled);
+    if (p.dtype == HQMQ_F16) return launch_layout<4, HQMQ_F16>(p, main_bits, flags, grid, st, tm, handled);
+    return launch_layout<4, HQMQ_BF16>(p, main_bits, flags, grid, st, tm, handled);
 }
 
 }  // namespace hqmq

@@ -225,8 +225,10 @@ def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int, ragged: bool =
 def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None, causal: bool = False,
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
-             force_generic: bool = False) -> torch.Tensor:
-    """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each)."""
+             force_generic: bool = False, kernel_events: Optional[tuple] = None) -> torch.Tensor:
+    """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each).
+    kernel_events: two raw hipEvent_t handles (ints) that receive the GPU timestamps of the begin and the end of
+    the main attention kernel (profiling)."""
     L.require_gpu(Q, "Q")
     if Q.stride(-1) != 1:
         Q = Q.contiguous()
@@ -260,6 +262,8 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     a.n_splits = n_splits
     a.skip_combine = int(skip_combine)
     a.force_generic = int(force_generic)
+    if kernel_events is not None:
+        a.start_event, a.stop_event = C.c_void_p(kernel_events[0]), C.c_void_p(kernel_events[1])
     ws = None
     if n_splits > 1:
         nbytes = int(L.lib().hqmq_attn_workspace_bytes(C.c_int(B), C.c_int(Hq), C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits)))

@@ -189,6 +189,8 @@ typedef struct hqmq_attn_args {
     void *workspace; int64_t workspace_bytes;
     int skip_combine;         /* 1: leave the split partials in the workspace (merge later with hqmq_attn_combine) */
     int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
+    void *start_event, *stop_event; /* hipEvent_t or NULL: receive the GPU timestamps of the begin and the end of
+                                       the main attention kernel (hipEventElapsedTime = its duration; profiling) */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
 /* The n_splits hqmq_attn_fwd would choose; ragged = 1 when kv_len is passed (more, smaller blocks). */
