@@ -397,6 +397,14 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     if (max(Kk, Kv) > FU * NT)
         fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
+    // Plain variants keep two half-steps in flight.  The second one is requested only now, when the table loads
+    // have come back: requested at the start it would queue in front of them and delay the whole block.
+    auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
+    FastTile<NW, AB, FLAGS, NH> tb;
+    if constexpr (!FLAGS) {
+        asm volatile("" ::: "memory");
+        load_super(readable(t_begin + 32 < t_end ? t_begin + 32 : t_begin), tb);
+    }
     if (FLAGS && threadIdx.x >= 64 && threadIdx.x < 100) {
         const uint32_t w = threadIdx.x - 64, row = w >> 2, d = w & 3;
         reinterpret_cast<uint32_t *>(lds_tab)[kSelOffset / 4 + w] = (row < 8 && (row >> 1) == d) ? 0x3C00u << (16 * (row & 1)) : 0u;
@@ -615,7 +623,28 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     VPre<kVPre> vc = {};
     if (FLAGS && t_begin < t_end) issue_all(f0, kc, vc);
 
-    for (int t0 = t_begin; t0 < t_end; t0 += STEP) {
+    if constexpr (!FLAGS) {
+        // ring of three tile buffers, every load unconditional (past the end the current tile is requested again)
+        FastTile<NW, AB, FLAGS, NH> tc;
+        int t0 = t_begin;
+        if (t0 < t_end) {
+            while (true) {
+                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), tc);
+                half_step(cur.h[0], t0, kc, vc);
+                t0 += 32;
+                if (t0 >= t_end) break;
+                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), cur);
+                half_step(tb.h[0], t0, kc, vc);
+                t0 += 32;
+                if (t0 >= t_end) break;
+                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), tb);
+                half_step(tc.h[0], t0, kc, vc);
+                t0 += 32;
+                if (t0 >= t_end) break;
+            }
+        }
+    }
+    for (int t0 = t_begin; FLAGS && t0 < t_end; t0 += STEP) {
         FastTile<NW, AB, FLAGS, NH> nxt;
         FlagTile f2 = {};
         KPre<kKPre> kn = {};
