@@ -44,6 +44,8 @@ def build(verbose: bool = False) -> Path:
         cmd = [cc, *COMMON, "-c", str(src), "-o", str(obj)]
         if src.name in EXACT:
             cmd.insert(1, "-ffp-contract=off")
+        if src.name == "quantize.hip":      # MFMA results straight into VGPRs: the search loop reads them at once
+            cmd[1:1] = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if verbose or r.returncode:
             sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)

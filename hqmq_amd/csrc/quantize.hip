@@ -68,6 +68,17 @@ __device__ __forceinline__ float best2_of(const float v[4]) {
     return fmaxf(mx + mx, sum);
 }
 
+// best2_of on the four results of the rotating MFMA, same values: |.| rides on the operands of v_max / v_max3
+// (the compiler's own code quiets every operand with an extra v_max first).  `sum` is also an input of the asm so
+// that it is placed behind the compiler's own first reads of the MFMA result.
+__device__ __forceinline__ float best2_mfma(float v0, float v1, float v2, float v3) {
+    const float sum = (fabsf(v0) + fabsf(v1)) + (fabsf(v2) + fabsf(v3));
+    float m23, mx;
+    asm("v_max_f32_e64 %0, |%1|, |%2|" : "=v"(m23) : "v"(v2), "v"(v3), "v"(sum));
+    asm("v_max3_f32 %0, |%1|, |%2|, %3" : "=v"(mx) : "v"(v0), "v"(v1), "v"(m23));
+    return fmaxf(mx + mx, sum);
+}
+
 // twice the exact score of Hurwitz unit p for rotated chunk v
 __device__ __forceinline__ float exact2_of(const float v[4], int p) {
     if (p < 8) {
@@ -187,12 +198,13 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
             // for every block, lane i holds column i), B = the lane's own direction, D = its rotated chunk.
             const half4 ub = half4{(_Float16)us[0], (_Float16)us[1], (_Float16)us[2], (_Float16)us[3]};
             const uint2 *acol = rot + (tid & 3);
+            uint2 a_next = acol[0];
             for (int s = 0; s < S; s++) {
-                const half4 am = __builtin_bit_cast(half4, acol[4 * s]);
+                const half4 am = __builtin_bit_cast(half4, a_next);
+                a_next = acol[4 * min(s + 1, S - 1)];           // the next column is on its way during this one
                 const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                const float v[4] = {vv[0], vv[1], vv[2], vv[3]};
-                const float b2 = best2_of(v);
-                m2 = fmaxf(m2, b2);
+                const float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
+                asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
                 if (b2 >= m2 - margin2) {
                     if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
                     cnt++;
@@ -275,7 +287,17 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
     // ---- per-token scale and radius code ----
     float rm = -INFINITY;
     bool rm_nan = false;
-    {
+    if ((n & (n - 1)) == 0 && n <= 64) {
+        // the n lanes of a token sit side by side inside one wavefront: butterfly over them
+        int bad = is_nan(r) ? 1 : 0;
+        rm = bad ? -INFINITY : r;
+        for (int o = 1; o < n; o <<= 1) {
+            const float other = __shfl_xor(rm, o, 64);
+            bad |= __shfl_xor(bad, o, 64);
+            rm = other > rm ? other : rm;
+        }
+        rm_nan = bad != 0;
+    } else {
         const int base = tok_local * n;
         for (int i = 0; i < n; i++) {
             float o = (base + i < kQThreads) ? radius_sh[base + i] : 0.f;
