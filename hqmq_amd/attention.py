@@ -3,9 +3,12 @@
 Signatures follow src/quantizers/hqmq_attention.py:68-75,425-438,
 hqmq_kernel.py:102-108, hqmq_attention_hopper.py:35-53,185-198 and
 hqmq_attention_blackwell.py:50-66 of the reference.  The Triton tuning knobs
-(block_q, block_kv, optimized, num_warps, num_stages, use_fp8_codebook) are
-accepted and ignored: there is one kernel, written for gfx950.  Extra keyword
-arguments (kv_lens, causal_offset, n_splits) are additions.
+(block_q, block_kv, optimized, num_warps, num_stages) are accepted and ignored:
+there is one kernel, written for gfx950.  use_fp8_codebook=True rounds the joint
+tables to float8_e4m3fn, as the reference's Hopper path does (there the fp8
+values are promoted to fp16 inside the kernel; here they are kept as fp16 in
+LDS, which is the same arithmetic).  Extra keyword arguments (kv_lens,
+causal_offset, n_splits) are additions.
 """
 from __future__ import annotations
 
@@ -53,6 +56,12 @@ def _pack_unpacked(idx, rq, rs, joint, r_qmax: int) -> PackedTensor:
     return pt
 
 
+def _through_fp8(joint: torch.Tensor) -> torch.Tensor:
+    """The table with every entry rounded to float8_e4m3fn, in its own dtype (every e4m3 number is exact in
+    fp16, bf16 and fp32)."""
+    return encode_joint_fp8(joint).to(joint.dtype)
+
+
 def fused_attention(
     Q: torch.Tensor,
     K_idx: torch.Tensor, K_radius_q: torch.Tensor, K_radius_scale: torch.Tensor, joint_K: torch.Tensor,
@@ -84,6 +93,8 @@ def fused_attention(
     if joint_K.shape[1] != joint_V.shape[1]:
         raise L.HqmqError("joint_K and joint_V must hold the same number of codewords")
     dt = joint_K.dtype
+    if use_fp8_codebook:
+        joint_K, joint_V = _through_fp8(joint_K), _through_fp8(joint_V)
     Qc = Q if Q.dtype == dt else Q.to(dt)
     Kc = _pack_unpacked(K_idx, K_radius_q, K_radius_scale, joint_K, r_qmax)
     Vc = _pack_unpacked(V_idx, V_radius_q, V_radius_scale, joint_V.to(dt), r_qmax)
@@ -95,14 +106,17 @@ def fused_attention(
 def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = False, softmax_scale: Optional[float] = None,
                            kv_lens: Optional[torch.Tensor] = None, causal_offset: int = 0, n_splits: int = 0,
                            T_kv: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                           force_generic: bool = False) -> torch.Tensor:
+                           force_generic: bool = False, use_fp8_codebook: bool = False) -> torch.Tensor:
     """Fused attention straight from the bit-packed cache (the fast path).
 
     Decode: T_q = 1, causal=False.  Chunked prefill: causal=True with causal_offset = number of
     cached tokens before the chunk (bottom-right alignment).  Ragged batches pass kv_lens (int32 [B]).
     force_generic runs the layout-generic kernel where a specialised one exists (a second implementation
-    of the same arithmetic, used by the tests).
+    of the same arithmetic, used by the tests).  use_fp8_codebook decodes with the joint tables rounded to
+    float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache).
     """
+    if use_fp8_codebook:
+        cache = PackedKV(cache.K.with_fp8_table(), cache.V.with_fp8_table())
     if T_kv is None:
         T_kv = cache.K.t_cap if kv_lens is not None else cache.K.length
     d, d_store = Q.shape[-1], cache.K.d_head
@@ -147,21 +161,21 @@ def fused_attention_reference(
 def fused_attention_hopper(Q, K_idx, K_radius_q, K_radius_scale, joint_K, V_idx, V_radius_q, V_radius_scale, joint_V,
                            r_qmax, causal=True, softmax_scale=None, block_q=256, block_kv=128, num_warps=8,
                            num_stages=3, use_fp8_codebook=True):
-    """Name kept for callers of the reference; runs the one gfx950 kernel (fp16 codebook in LDS)."""
+    """Name kept for callers of the reference; runs the one gfx950 kernel (fp8 table by default, as there)."""
     return fused_attention(Q, K_idx, K_radius_q, K_radius_scale, joint_K, V_idx, V_radius_q, V_radius_scale, joint_V,
-                           r_qmax, causal=causal, softmax_scale=softmax_scale)
+                           r_qmax, causal=causal, softmax_scale=softmax_scale, use_fp8_codebook=use_fp8_codebook)
 
 
 def fused_attention_blackwell(Q, K_idx, K_radius_q, K_radius_scale, joint_K, V_idx, V_radius_q, V_radius_scale, joint_V,
                               r_qmax, causal=True, softmax_scale=None, block_q=256, block_kv=256, num_warps=8,
                               num_stages=4, use_fp8_codebook=True):
-    """Name kept for callers of the reference; runs the one gfx950 kernel."""
+    """Name kept for callers of the reference; runs the one gfx950 kernel (fp8 table by default, as there)."""
     return fused_attention(Q, K_idx, K_radius_q, K_radius_scale, joint_K, V_idx, V_radius_q, V_radius_scale, joint_V,
-                           r_qmax, causal=causal, softmax_scale=softmax_scale)
+                           r_qmax, causal=causal, softmax_scale=softmax_scale, use_fp8_codebook=use_fp8_codebook)
 
 
 def encode_joint_fp8(joint_fp16: torch.Tensor) -> torch.Tensor:
-    """(H, K, 4) joint codebook -> float8_e4m3fn (storage format only; the kernels gather fp16)."""
+    """(H, K, 4) joint codebook -> float8_e4m3fn."""
     return joint_fp16.to(torch.float8_e4m3fn)
 
 
@@ -185,4 +199,4 @@ def device_info() -> dict:
     arch = getattr(props, "gcnArchName", "").split(":")[0]
     return {"gpu": torch.cuda.get_device_name(), "compute_capability": f"{cap[0]}.{cap[1]}", "arch": arch,
             "variant": "cdna4", "variant_auto_dispatched": "cdna4", "fp8_codebook": False,
-            "fp8_codebook_supported": False}
+            "fp8_codebook_supported": True}

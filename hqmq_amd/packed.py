@@ -120,6 +120,20 @@ class PackedTensor:
         dropped = torch.arange(self.t_cap, device=self.device).view(1, 1, self.t_cap, 1) >= lens.view(B, 1, 1, 1)
         self.flags.masked_fill_(dropped, 0)                # no flag without an entry behind it
 
+    def with_fp8_table(self) -> "PackedTensor":
+        """A view of the same planes whose joint table is rounded to float8_e4m3fn (kept in the table's dtype:
+        every e4m3 number is exact there).  The rounded table is computed once per table."""
+        import copy
+        cached = getattr(self, "_fp8_view", None)
+        if cached is None or cached[0] is not self.joint:
+            view = copy.copy(self)
+            view.joint = self.joint.to(torch.float8_e4m3fn).to(self.joint.dtype)
+            cached = (self.joint, view)
+            self._fp8_view = cached
+        view = cached[1]
+        view.length, view.lengths = self.length, self.lengths
+        return view
+
     def check_overflow(self) -> None:
         """Raises if an append ran out of sideband room (reads one int from the device)."""
         if self.sb_overflow is not None and int(self.sb_overflow.item()):

@@ -42,9 +42,13 @@ def test_device_info_reports_real_gpu():
     assert info["arch"].startswith("gfx950")
 
 
-def test_fp8_flag_is_ignored():
-    """use_fp8_codebook=True falls through to the same kernel (the reference's pre-Hopper behaviour)."""
+def test_fp8_codebook_option():
+    """use_fp8_codebook=True is the reference's Hopper behaviour: the joint tables rounded to float8_e4m3fn, fp16
+    arithmetic.  It equals the plain call on the rounded tables bit for bit, dense attention over a cache decoded
+    with them within the usual bound, and it is the default of the hopper / blackwell names."""
     import hqmq
+    from hqmq import kernels
+    from hqmq_amd import ops
     B, H_q, H_kv, T, dh, S, r_qmax = 1, 4, 1, 32, 32, 24, 7
     torch.manual_seed(0)
     Q = torch.randn(B, H_q, T, dh, dtype=torch.float16, device="cuda") * 0.3
@@ -53,13 +57,37 @@ def test_fp8_flag_is_ignored():
     rs = torch.rand((B, H_kv, T), dtype=torch.float16, device="cuda") + 0.5
     joint = torch.randn((H_kv, 24 * S, 4), dtype=torch.float16, device="cuda")
     joint = joint / joint.norm(dim=-1, keepdim=True).clamp(min=1e-6)
+    j8 = kernels.encode_joint_fp8(joint).to(torch.float16)
+    assert not torch.equal(j8, joint)
     a = hqmq.fused_attention(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
     b = hqmq.fused_attention(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True, use_fp8_codebook=True)
-    assert torch.equal(a, b)
-    from hqmq import kernels
+    on_rounded = hqmq.fused_attention(Q, idx, rq, rs, j8, idx, rq, rs, j8, r_qmax=r_qmax, causal=True)
+    assert torch.equal(b, on_rounded) and not torch.equal(a, b)
+    ref = hqmq.fused_attention_reference(Q, idx, rq, rs, j8, idx, rq, rs, j8, r_qmax=r_qmax, causal=True)
+    assert (b.float() - ref.float()).abs().max().item() < 2e-3
     c = kernels.fused_attention_hopper(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
-    d = kernels.fused_attention_blackwell(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True)
-    assert torch.equal(a, c) and torch.equal(a, d)
+    d = kernels.fused_attention_blackwell(Q, idx, rq, rs, joint, idx, rq, rs, joint, r_qmax=r_qmax, causal=True,
+                                          use_fp8_codebook=False)
+    assert torch.equal(b, c) and torch.equal(a, d)
+    # the packed path: same option, per cache
+    q = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=2, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    g = torch.Generator().manual_seed(5)
+    k, v = torch.randn(2, 2, 100, 128, generator=g).half().to(DEV), torch.randn(2, 2, 100, 128, generator=g).half().to(DEV)
+    k[:, :, ::9, 8:12] *= 30.0
+    cache = q.new_cache(2, 100, 128, torch.float16, 0)
+    q.append(cache, k, v, 0)
+    Qp = torch.randn(2, 8, 1, 128, generator=g).half().to(DEV)
+    table_before = cache.K.joint.clone()
+    O8 = hqmq.fused_attention_packed(Qp, cache, use_fp8_codebook=True)
+    O16 = hqmq.fused_attention_packed(Qp, cache)
+    from hqmq_amd.packed import PackedKV
+    view = PackedKV(cache.K.with_fp8_table(), cache.V.with_fp8_table())
+    Kd = ops.dequant_packed(view.K, 100, 0).float().repeat_interleave(4, 1)
+    Vd = ops.dequant_packed(view.V, 100, 0).float().repeat_interleave(4, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Qp.float(), Kd) * 128 ** -0.5
+    refp = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
+    assert (O8.float() - refp).abs().max().item() < 2e-3 * max(1.0, float(refp.abs().max()))
+    assert not torch.equal(O8, O16) and torch.equal(cache.K.joint, table_before)      # the cache keeps its own table
 
 
 def test_encode_joint_fp8():

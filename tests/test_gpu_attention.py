@@ -36,7 +36,7 @@ def test_golden_unpacked_api(case, golden_dir):
     d = {k: v.to(DEV) for k, v in t.items()}
     base = 1e-3 if m["dtype"] == torch.float32 else 2e-3
     for kw in (dict(), dict(n_splits=1), dict(n_splits=3), dict(block_q=64, block_kv=64, num_warps=4, num_stages=2,
-                                                               optimized=False, use_fp8_codebook=True)):
+                                                               optimized=False)):
         O = hqmq.fused_attention(d["Q"], d["K_idx"], d["K_rq"], d["K_rs"], d["K_joint"], d["V_idx"], d["V_rq"],
                                  d["V_rs"], d["V_joint"], r_qmax=m["qmax"], causal=m["causal"], **kw)
         assert O.shape == d["Q"].shape and O.dtype == d["Q"].dtype
