@@ -81,9 +81,12 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     const int col_lim = (int)lim64;
     int blk_lim = col_lim;                        // block-wide limit: max over the 16 columns
     for (int o = 1; o < 16; o <<= 1) blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
-    int per_split = (blk_lim + p.n_splits - 1) / p.n_splits;
+    // tokens before kv_start[b] are invisible (left padding): the walk starts at the super-tile that holds it
+    const int col_start = p.kv_start ? min(max(p.kv_start[b], 0), blk_lim) : 0;
+    const int blk_lo = col_start / kSuper * kSuper;
+    int per_split = (blk_lim - blk_lo + p.n_splits - 1) / p.n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
-    const int b_begin = min(sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
+    const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
     int per_wave = (b_end - b_begin + kAttnWaves - 1) / kAttnWaves;
     per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
@@ -191,7 +194,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
                 const int t = t0 + 16 * u + 4 * grp + e;
                 float v = sT[u][e] * (cur.ks[u][e] * p.c_log2);
                 if (FLAGS) v = fmaf(sTo[u][e], p.c_plain, v);
-                v = (t < col_lim && t < t_end) ? v : -INFINITY;
+                v = (t < col_lim && t < t_end && t >= col_start) ? v : -INFINITY;
                 pv[u][e] = v;
                 tmax = fmaxf(tmax, v);
             }
@@ -453,7 +456,7 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     p.B = a->B; p.Hq = a->H_q; p.Hkv = a->H_kv; p.G = a->H_q / a->H_kv; p.Tq = a->T_q; p.Tkv = a->T_kv; p.n = n;
     p.t_cap = a->t_cap;
     p.idx_bits = a->idx_bits; p.aux_bits = a->aux_bits; p.qmax = a->qmax;
-    p.kv_len = a->kv_len; p.causal = a->causal; p.causal_offset = a->causal_offset;
+    p.kv_len = a->kv_len; p.kv_start = a->kv_start; p.causal = a->causal; p.causal_offset = a->causal_offset;
     p.c_log2 = a->softmax_scale * 1.4426950408889634f / (float)a->qmax;
     p.c_plain = a->softmax_scale * 1.4426950408889634f;
     p.inv_qmax = 1.0f / (float)a->qmax;

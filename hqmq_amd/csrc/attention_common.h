@@ -35,6 +35,7 @@ struct AttnParams {
     int64_t t_cap;
     int idx_bits, aux_bits, qmax;
     const int32_t *kv_len;
+    const int32_t *kv_start;   // [B] or NULL: the first visible token of every sequence (left padding)
     int causal;
     int64_t causal_offset;
     float c_log2;   // softmax_scale * log2(e) / qmax

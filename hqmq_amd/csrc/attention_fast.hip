@@ -282,9 +282,12 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
     blk_lim = __builtin_amdgcn_readfirstlane(blk_lim);      // the same in every lane: all rows hold all 16 columns
     lim_min = __builtin_amdgcn_readfirstlane(lim_min);
-    int per_split = (blk_lim + p.n_splits - 1) / p.n_splits;
+    // tokens before kv_start[b] are invisible (left padding): the walk starts at the super-tile that holds it
+    const int col_start = p.kv_start ? min(max(p.kv_start[b], 0), blk_lim) : 0;
+    const int blk_lo = col_start / kSuper * kSuper;
+    int per_split = (blk_lim - blk_lo + p.n_splits - 1) / p.n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
-    const int b_begin = min(sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
+    const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
     int per_wave = (b_end - b_begin + kFastWaves - 1) / kFastWaves;
     per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
     // every super-tile starts at a multiple of 64 below T_kv <= t_cap (a multiple of 64): whole tiles are readable
@@ -563,13 +566,13 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
             sT[u] = s;
         }
         // ---- mask (boundary half-steps only), online softmax ----
-        if (!(th + 32 <= lim_min && th + 32 <= t_end)) {
+        if (!(th + 32 <= lim_min && th + 32 <= t_end && th >= col_start)) {
 #pragma unroll
             for (int u = 0; u < 2; u++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int t = th + 16 * u + 4 * grp + e;
-                    if (!(t < col_lim && t < t_end)) sT[u][e] = -INFINITY;
+                    if (!(t < col_lim && t < t_end && t >= col_start)) sT[u][e] = -INFINITY;
                 }
         }
         float tmax = fmaxf(fmaxf(fmaxf(sT[0][0], sT[0][1]), fmaxf(sT[0][2], sT[0][3])),

@@ -14,8 +14,8 @@ PackedQuantizedCache  +  attn_implementation="hqmq_packed"
     cache = PackedQuantizedCache(quantizer, max_tokens=4096)
     out = model(input_ids, past_key_values=cache, use_cache=True)
 
-Limits: unpadded batches (every sequence of the batch has the same length; the causal mask is the only mask),
-no beam reordering (cropping is supported).  This module imports `transformers`; nothing else in the package does.
+Limits: the mask is causal, optionally with left padding (the usual batched-generation layout; pad tokens are
+quantized and stored like any other, and never attended to); no beam reordering (cropping is supported).  This module imports `transformers`; nothing else in the package does.
 """
 from __future__ import annotations
 
@@ -130,8 +130,19 @@ def hqmq_packed_attention(module, query, key, value, attention_mask, dropout: fl
         raise NotImplementedError("attention dropout is not supported on the packed path")
     t_q = query.shape[2]
     out = fused_attention_packed(query, layer.packed, causal=True, causal_offset=layer.n_tokens - t_q,
-                                 softmax_scale=scaling, T_kv=layer.n_tokens)
+                                 softmax_scale=scaling, T_kv=layer.n_tokens,
+                                 kv_starts=_first_visible(attention_mask, layer.n_tokens))
     return out.transpose(1, 2).contiguous(), None
+
+
+def _first_visible(attention_mask, t_kv: int):
+    """Left padding from the 4-D mask the model built (bool, or additive with 0 = visible): the first key the
+    last query row may see, per sequence.  Everything else about the mask is taken to be causal."""
+    if attention_mask is None:
+        return None
+    row = attention_mask[:, 0, -1, :t_kv]
+    visible = row if row.dtype == torch.bool else row > -1.0
+    return visible.to(torch.int32).argmax(-1).to(torch.int32)
 
 
 def register() -> str:

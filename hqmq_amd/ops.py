@@ -222,7 +222,8 @@ def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int, ragged: bool =
                                              C.c_int(1 if ragged else 0)))
 
 
-def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None, causal: bool = False,
+def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None,
+             kv_starts: Optional[torch.Tensor] = None, causal: bool = False,
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
              force_generic: bool = False, kernel_events: Optional[tuple] = None) -> torch.Tensor:
@@ -258,6 +259,12 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     if kv_lens is not None:
         keep = kv_lens.to(device=dev, dtype=torch.int32).contiguous()
         a.kv_len = L.ptr(keep)
+    keep_start = None
+    if kv_starts is not None:
+        keep_start = kv_starts.to(device=dev, dtype=torch.int32).contiguous()
+        if keep_start.numel() != B:
+            raise L.HqmqError(f"kv_starts must hold one entry per sequence ({B})")
+        a.kv_start = L.ptr(keep_start)
     a.causal, a.causal_offset, a.softmax_scale = int(causal), causal_offset, softmax_scale
     a.n_splits = n_splits
     a.skip_combine = int(skip_combine)

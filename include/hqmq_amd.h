@@ -189,6 +189,7 @@ typedef struct hqmq_attn_args {
     void *workspace; int64_t workspace_bytes;
     int skip_combine;         /* 1: leave the split partials in the workspace (merge later with hqmq_attn_combine) */
     int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
+    const int32_t *kv_start;  /* [B] or NULL: first visible token of every sequence (left-padded batches) */
     void *start_event, *stop_event; /* hipEvent_t or NULL: receive the GPU timestamps of the begin and the end of
                                        the main attention kernel (hipEventElapsedTime = its duration; profiling) */
 } hqmq_attn_args;

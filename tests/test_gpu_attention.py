@@ -384,3 +384,41 @@ def test_crop_per_sequence_then_decode_appends():
     for generic in (False, True):
         O = hqmq.fused_attention_packed(Q, cache, causal=False, kv_lens=pos, T_kv=Tm, force_generic=generic)
         assert (O.float() - ref).abs().max().item() < tol, generic
+
+
+@pytest.mark.parametrize("med3x,Tq", [(False, 1), (True, 1), (True, 24)])
+def test_left_padded_batch(med3x, Tq):
+    """kv_starts: the tokens in front of every sequence's first real one are invisible (left padding), decode and
+    chunked prefill, both kernels, against dense attention with the explicit mask."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.float16
+    B, Hq, Hkv, T, d_h = 4, 8, 2, 300, 128
+    if med3x:
+        k, v = _planted(B, Hkv, T, d_h, 31, dt), _planted(B, Hkv, T, d_h, 32, dt)
+    else:
+        g = torch.Generator().manual_seed(31)
+        k, v = torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV)
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV)
+    w = hqmq.with_outlier_extraction(q, C=3.0) if med3x else q
+    cache = w.new_cache(B, T, d_h, dt, 0, **({"sideband_frac": 0.5} if med3x else {}))
+    w.append(cache, k, v, 0)
+    starts = torch.tensor([0, 7, 64, 201], dtype=torch.int32, device=DEV)
+    Q = torch.randn(B, Hq, Tq, d_h, generator=torch.Generator().manual_seed(33)).to(dt).to(DEV)
+    off = T - Tq
+    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    kk = torch.arange(T, device=DEV).view(1, 1, 1, T)
+    mask = (kk <= torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off) & (kk >= starts.view(B, 1, 1, 1))
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
+    tol = 2e-3 * max(1.0, float(ref.abs().max()))
+    for generic in (False, True):
+        for ns in (0, 1, 3):
+            O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, kv_starts=starts, n_splits=ns,
+                                            force_generic=generic)
+            assert (O.float() - ref).abs().max().item() < tol, (generic, ns)
+    # a start behind everything a query may see: that row attends to nothing and comes back as zeros
+    late = torch.full((B,), T, dtype=torch.int32, device=DEV)
+    O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, kv_starts=late)
+    assert int(O.abs().sum()) == 0

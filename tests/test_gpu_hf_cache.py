@@ -96,3 +96,42 @@ def test_packed_cache_crop_replays_identically():
     cache.check_overflow()
     assert cache.get_seq_length() == 146 and torch.equal(once[2:], again)
     assert [int(layer.packed.K.sb_count.sum()) for layer in cache.layers] == counts
+
+
+def test_left_padded_generation_batch():
+    """Sequences of different lengths, left-padded as generate() lays them out: the packed cache + fused attention
+    follow the fake-quantizing cache + sdpa on the real positions, prefill and decode steps."""
+    import hqmq
+    from src.model_utils import ATTN_NAME, PackedQuantizedCache, QuantizedCache
+    dt = torch.float16
+    model = tiny_llama(dt)
+    q = hqmq.HQMQ(n_layers=3, n_heads=2, secondary_size=96, radius_bits=4, device=DEV)
+    B, T, steps = 3, 90, 4
+    pads = [0, 13, 40]
+    ids = torch.randint(1, 256, (B, T + steps), generator=torch.Generator().manual_seed(3)).to(DEV)
+    mask = torch.ones(B, T + steps, dtype=torch.long, device=DEV)
+    for b, p in enumerate(pads):
+        mask[b, :p] = 0
+        ids[b, :p] = 0
+    pos = (mask.cumsum(-1) - 1).clamp(min=0)
+
+    def run(cache):
+        logits = []
+        with torch.no_grad():
+            out = model(ids[:, :T], attention_mask=mask[:, :T], position_ids=pos[:, :T], past_key_values=cache, use_cache=True)
+            logits.append(out.logits[:, -1].float())
+            for s in range(steps):
+                out = model(ids[:, T + s:T + s + 1], attention_mask=mask[:, :T + s + 1], position_ids=pos[:, T + s:T + s + 1],
+                            past_key_values=cache, use_cache=True)
+                logits.append(out.logits[:, -1].float())
+        return torch.stack(logits)
+
+    model.set_attn_implementation("sdpa")
+    want = run(QuantizedCache(q))
+    model.set_attn_implementation(ATTN_NAME)
+    packed = PackedQuantizedCache(q, max_tokens=128)
+    got = run(packed)
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    print(f"left-padded batch: max|logit| {scale:.3f}, packed vs fake-quant {err:.2e}")
+    assert err < 0.02 * scale, (err, scale)
