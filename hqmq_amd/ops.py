@@ -109,7 +109,8 @@ _WS = {}
 
 def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
     """A cached scratch buffer of at least nbytes (grown on demand, reused across calls)."""
-    key = (tag, torch.device(device))
+    dev = torch.device(device)
+    key = (tag, dev, torch.cuda.current_stream(dev).cuda_stream)     # calls on different streams may overlap
     buf = _WS.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)   # attention counters start at zero
