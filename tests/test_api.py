@@ -203,3 +203,42 @@ def test_memory_table_uses_packed_layout():
     for S, b in MT.CONFIGS:
         k = f"hqmq_s{S}_r{b}"
         assert r[k + "_analytic_MB"] <= r[k + "_MB"] <= 1.08 * r[k + "_analytic_MB"]
+
+
+def test_crop_bookkeeping_on_cpu():
+    """PackedTensor.crop_ is plain torch: after a crop, the entry count and the tile offsets equal what appending
+    only the kept rows would have left, and no flag stays behind in a dropped row."""
+    import numpy as np
+    from hqmq_amd.packed import PackedTensor, TILE
+    rng = np.random.default_rng(0)
+    B, H, T, d_h = 3, 2, 150, 64
+    n = d_h // 4
+    pt = PackedTensor(B, H, T, d_h, 96, 4, torch.float16, "cpu", outliers=True, sideband_frac=1.0)
+    bits = rng.random((B, H, T, n)) < 0.07
+    flags = np.zeros((B, H, pt.t_cap, n // 8), np.uint8)
+    for c in range(n):
+        flags[:, :, :T, c // 8] |= (bits[..., c].astype(np.uint8) << (c % 8))
+    per_row = bits.sum(-1)                                             # (B, H, T)
+
+    def state(lengths):                                                # what in-order appends of `lengths` rows leave
+        off = np.full((B, H, pt.t_cap // TILE), 0x7fffffff, np.int64)
+        cnt = np.zeros((B, H), np.int64)
+        for b in range(B):
+            for t in range(-(-lengths[b] // TILE)):
+                off[b, :, t] = per_row[b, :, :t * TILE].sum(-1)
+            cnt[b] = per_row[b, :, :lengths[b]].sum(-1)
+        return off, cnt
+    off, cnt = state([T] * B)
+    pt.flags.copy_(torch.from_numpy(flags))
+    pt.sb_tile_off.copy_(torch.from_numpy(off).to(torch.int32))
+    pt.sb_count.copy_(torch.from_numpy(cnt).to(torch.int32))
+    pt.length = T
+    lens = [150, 96, 37]                                               # no-op, tile-aligned, inside a tile
+    pt.crop_(torch.tensor(lens, dtype=torch.int32))
+    off2, cnt2 = state(lens)
+    assert np.array_equal(pt.sb_count.numpy(), cnt2) and np.array_equal(pt.sb_tile_off.numpy(), off2)
+    for b in range(B):
+        assert int(pt.flags[b, :, lens[b]:].sum()) == 0 and np.array_equal(pt.flags[b, :, :lens[b]].numpy(), flags[b, :, :lens[b]])
+    pt.crop_(20)                                                       # an int crops every sequence
+    off3, cnt3 = state([20] * B)
+    assert pt.length == 20 and np.array_equal(pt.sb_count.numpy(), cnt3) and np.array_equal(pt.sb_tile_off.numpy(), off3)
