@@ -57,7 +57,7 @@ class AttnArgs(C.Structure):
         ("idx_bits", C.c_int), ("main_bits", C.c_int), ("aux_bits", C.c_int), ("qmax", C.c_int),
         ("kv_len", vp), ("causal", C.c_int), ("causal_offset", i64), ("softmax_scale", C.c_float),
         ("n_splits", C.c_int), ("workspace", vp), ("workspace_bytes", i64), ("skip_combine", C.c_int), ("force_generic", C.c_int),
-        ("kv_start", vp), ("start_event", vp), ("stop_event", vp),
+        ("kv_start", vp), ("batch_order", vp), ("start_event", vp), ("stop_event", vp),
     ]
 
 

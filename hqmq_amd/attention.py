@@ -107,12 +107,14 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
                            kv_lens: Optional[torch.Tensor] = None, causal_offset: int = 0, n_splits: int = 0,
                            T_kv: Optional[int] = None, out: Optional[torch.Tensor] = None,
                            force_generic: bool = False, use_fp8_codebook: bool = False,
-                           kv_starts: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           kv_starts: Optional[torch.Tensor] = None,
+                           batch_order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Fused attention straight from the bit-packed cache (the fast path).
 
     Decode: T_q = 1, causal=False.  Chunked prefill: causal=True with causal_offset = number of
     cached tokens before the chunk (bottom-right alignment).  Ragged batches pass kv_lens (int32 [B]);
-    left-padded batches pass kv_starts (int32 [B], the first real token of every sequence).
+    left-padded batches pass kv_starts (int32 [B], the first real token of every sequence).  batch_order (int32 [B],
+    e.g. ops.longest_first(kv_lens)) starts the sequences' blocks in that order: scheduling only, same result.
     force_generic runs the layout-generic kernel where a specialised one exists (a second implementation
     of the same arithmetic, used by the tests).  use_fp8_codebook decodes with the joint tables rounded to
     float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache).
@@ -127,14 +129,14 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
         if softmax_scale is None:
             softmax_scale = d ** -0.5
         O = ops.attn_fwd(torch.nn.functional.pad(Q, (0, d_store - d)), cache.K, cache.V, T_kv, kv_lens=kv_lens,
-                         kv_starts=kv_starts, causal=causal,
+                         kv_starts=kv_starts, batch_order=batch_order, causal=causal,
                          causal_offset=causal_offset, softmax_scale=softmax_scale, n_splits=n_splits,
                          force_generic=force_generic)[..., :d]
         if out is not None:
             out.copy_(O)
             return out
         return O.contiguous()
-    return ops.attn_fwd(Q, cache.K, cache.V, T_kv, kv_lens=kv_lens, kv_starts=kv_starts, causal=causal,
+    return ops.attn_fwd(Q, cache.K, cache.V, T_kv, kv_lens=kv_lens, kv_starts=kv_starts, batch_order=batch_order, causal=causal,
                         causal_offset=causal_offset, softmax_scale=softmax_scale, n_splits=n_splits, out=out,
                         force_generic=force_generic)
 

@@ -128,8 +128,11 @@ def run(cfg, steps):
     step_bytes = 2 * Hkv * tokens * row + flagged * 4 * cache.K.scale.element_size()
     n_splits = ops.pick_splits(B, Hq, Hkv, 1, T if lens is None else int(lens.max()), lens is not None)
 
+    # ragged batch: the longest sequences start first (the order holds while all contexts grow in step)
+    order = ops.longest_first(lens_dev) if lens is not None else None
+
     def attend():
-        hqmq.fused_attention_packed(Q, cache, kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out)
+        hqmq.fused_attention_packed(Q, cache, kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
     us = event_us(attend, steps)
     res = {"config": name, "us_per_step": round(us, 2), "compressed_bytes_per_step": step_bytes,
            "GBps": round(step_bytes / us / 1e3, 1), "pct_of_hbm_roofline": round(100 * step_bytes / us / 1e3 / HBM_PEAK_GBPS, 2),
@@ -148,7 +151,7 @@ def run(cfg, steps):
 
         def step():
             append()
-            hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T, n_splits=n_splits, out=out)
+            hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
         res["us_per_step_with_append"] = round(event_us(step, steps), 2)
         res["us_append_only"] = round(event_us(append, steps), 2)
         # the same step replayed from a HIP graph: what the GPU needs once the ten small launches of an append are

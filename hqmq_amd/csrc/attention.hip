@@ -61,7 +61,11 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + p.Kc.K;
 
-    const int bh = blockIdx.z, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
+    // blocks are dispatched in grid order: batch_order lists the sequences in the order they should start
+    // (longest first for ragged batches, so that no long sequence is left for the end)
+    const int slot = blockIdx.z / p.Hkv, hkv = blockIdx.z - slot * p.Hkv;
+    const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
+    const int bh = b * p.Hkv + hkv;
     const int cg = blockIdx.y, sp = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int dtype = p.dtype;
@@ -456,7 +460,7 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
     p.B = a->B; p.Hq = a->H_q; p.Hkv = a->H_kv; p.G = a->H_q / a->H_kv; p.Tq = a->T_q; p.Tkv = a->T_kv; p.n = n;
     p.t_cap = a->t_cap;
     p.idx_bits = a->idx_bits; p.aux_bits = a->aux_bits; p.qmax = a->qmax;
-    p.kv_len = a->kv_len; p.kv_start = a->kv_start; p.causal = a->causal; p.causal_offset = a->causal_offset;
+    p.kv_len = a->kv_len; p.kv_start = a->kv_start; p.batch_order = a->batch_order; p.causal = a->causal; p.causal_offset = a->causal_offset;
     p.c_log2 = a->softmax_scale * 1.4426950408889634f / (float)a->qmax;
     p.c_plain = a->softmax_scale * 1.4426950408889634f;
     p.inv_qmax = 1.0f / (float)a->qmax;

@@ -36,6 +36,7 @@ struct AttnParams {
     int idx_bits, aux_bits, qmax;
     const int32_t *kv_len;
     const int32_t *kv_start;   // [B] or NULL: the first visible token of every sequence (left padding)
+    const int32_t *batch_order; // [B] or NULL: a permutation of the sequences, the order their blocks start in
     int causal;
     int64_t causal_offset;
     float c_log2;   // softmax_scale * log2(e) / qmax

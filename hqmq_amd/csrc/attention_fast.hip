@@ -253,12 +253,16 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = kFastWaves * 64;
-    constexpr int kKPre = CPL >= 8 ? 2 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
+    constexpr int kKPre = CPL >= 8 ? 3 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
 
-    const int bh = blockIdx.z, b = bh / p.Hkv, hkv = bh - b * p.Hkv;
+    // blocks are dispatched in grid order: batch_order lists the sequences in the order they should start
+    // (longest first for ragged batches, so that no long sequence is left for the end)
+    const int slot = blockIdx.z / p.Hkv, hkv = blockIdx.z - slot * p.Hkv;
+    const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
+    const int bh = b * p.Hkv + hkv;
     const int cg = blockIdx.y, sp = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int G = p.G;

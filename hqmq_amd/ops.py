@@ -223,8 +223,14 @@ def pick_splits(B: int, H_q: int, H_kv: int, T_q: int, T_kv: int, ragged: bool =
                                              C.c_int(1 if ragged else 0)))
 
 
+def longest_first(kv_lens: torch.Tensor) -> torch.Tensor:
+    """The batch_order for a ragged batch: sequences sorted by length, longest first (int32, on kv_lens' device).
+    It stays valid while all sequences grow in step, so a decode loop computes it once."""
+    return torch.argsort(kv_lens, descending=True, stable=True).to(torch.int32)
+
+
 def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tensor] = None,
-             kv_starts: Optional[torch.Tensor] = None, causal: bool = False,
+             kv_starts: Optional[torch.Tensor] = None, batch_order: Optional[torch.Tensor] = None, causal: bool = False,
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
              force_generic: bool = False, kernel_events: Optional[tuple] = None) -> torch.Tensor:
@@ -266,6 +272,12 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
         if keep_start.numel() != B:
             raise L.HqmqError(f"kv_starts must hold one entry per sequence ({B})")
         a.kv_start = L.ptr(keep_start)
+    keep_order = None
+    if batch_order is not None:
+        keep_order = batch_order.to(device=dev, dtype=torch.int32).contiguous()
+        if keep_order.numel() != B:
+            raise L.HqmqError(f"batch_order must be a permutation of the {B} sequences")
+        a.batch_order = L.ptr(keep_order)
     a.causal, a.causal_offset, a.softmax_scale = int(causal), causal_offset, softmax_scale
     a.n_splits = n_splits
     a.skip_combine = int(skip_combine)

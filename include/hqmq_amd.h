@@ -190,6 +190,8 @@ typedef struct hqmq_attn_args {
     int skip_combine;         /* 1: leave the split partials in the workspace (merge later with hqmq_attn_combine) */
     int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
     const int32_t *kv_start;  /* [B] or NULL: first visible token of every sequence (left-padded batches) */
+    const int32_t *batch_order; /* [B] or NULL: a permutation of 0..B-1, the order in which the sequences' blocks are
+                                   started (pass the sequences sorted by length, longest first, for ragged batches) */
     void *start_event, *stop_event; /* hipEvent_t or NULL: receive the GPU timestamps of the begin and the end of
                                        the main attention kernel (hipEventElapsedTime = its duration; profiling) */
 } hqmq_attn_args;

@@ -422,3 +422,25 @@ def test_left_padded_batch(med3x, Tq):
     late = torch.full((B,), T, dtype=torch.int32, device=DEV)
     O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, kv_starts=late)
     assert int(O.abs().sum()) == 0
+
+
+def test_batch_order_is_scheduling_only():
+    """batch_order changes which sequence's blocks start first, never the result: bit-equal outputs for the natural
+    order, longest-first and a shuffled permutation, ragged batch with outliers, both kernels."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.bfloat16
+    B, Hq, Hkv, T, d_h = 6, 8, 2, 260, 128
+    k, v = _planted(B, Hkv, T, d_h, 41, dt), _planted(B, Hkv, T, d_h, 42, dt)
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=24, radius_bits=3, device=DEV), C=3.0)
+    cache = w.new_cache(B, T, d_h, dt, 0, sideband_frac=0.5)
+    w.append(cache, k, v, 0)
+    lens = torch.tensor([260, 17, 128, 255, 1, 64], dtype=torch.int32, device=DEV)
+    Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(43)).to(dt).to(DEV)
+    lf = ops.longest_first(lens)
+    assert lf.tolist() == [0, 3, 2, 5, 1, 4]
+    for generic in (False, True):
+        base = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=2, force_generic=generic)
+        for order in (lf, torch.tensor([4, 2, 0, 5, 3, 1], dtype=torch.int32, device=DEV)):
+            O = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=2, force_generic=generic, batch_order=order)
+            assert torch.equal(O, base)
