@@ -11,8 +11,8 @@
 //   O^T += V^T . P^T  v_mfma_f32_16x16x32_f16 over two tiles (32 tokens) at a time.
 // Row j of the V-side product is d = (grp * CPL + j) * 4 + e, the order the epilogue writes back.
 // Scores are kept as S^T * rs; 1/qmax is folded into the softmax scale and the epilogue.  Outlier chunks
-// (flag bit set) carry radius code 0, so they decode to zero, and enter through extra MFMAs with their
-// verbatim sideband values.
+// carry radius code 0 in the planes, so they decode to zero; their verbatim values enter through extra MFMAs
+// that walk the sideband entry list (values + coordinates), never the flag plane.
 #include "attention_common.h"
 
 namespace hqmq {
@@ -229,15 +229,6 @@ __device__ __forceinline__ float row_sum4(float x) {
     return __uint_as_float(q[0]) + __uint_as_float(q[1]);
 }
 
-// inclusive prefix sum over the 16 lanes of a row (DPP row_shr with zero fill)
-__device__ __forceinline__ int row_prefix16(int x) {
-    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, true);
-    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, true);
-    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, true);
-    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, true);
-    return x;
-}
-
 // fp32 4-vector (exact fp16 values) -> packed fp16
 __device__ __forceinline__ half4 pack4(float4v t) {
     const auto lo = __builtin_amdgcn_cvt_pkrtz(t[0], t[1]);
@@ -298,7 +289,7 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
 
     const size_t plane_row0 = (size_t)bh * p.t_cap;
-    constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8, frb = (n + 7) / 8;
+    constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8;
     const int64_t tiles_cap = p.t_cap / kTile;
     const int tiles_cap1 = (int)tiles_cap - 1;
     const int idx_bits = p.idx_bits;
