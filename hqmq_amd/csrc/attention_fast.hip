@@ -51,7 +51,7 @@ __device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, in
     }
 }
 
-constexpr int kFastWaves = 8;
+constexpr int kFastWaves = 8;     // wavefronts per block; 12 (three per SIMD) for plain 16+0 caches with long ranges per block
 
 // codes, aux bits and raw 16-bit scales of 32 tokens (two 16-token tiles) for one lane
 template <int NW, int AB, bool FLAGS>
@@ -236,14 +236,14 @@ __device__ __forceinline__ half4 pack4(float4v t) {
     return __builtin_bit_cast(half4, uint2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)});
 }
 
-template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS>
-__global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParams p) {
+template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS, int WV = kFastWaves>
+__global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(AttnParams p) {
     constexpr int NB = CPL * MB / 8;
     constexpr int NW = (NB + 3) / 4;
     constexpr int ABYTES = CPL * AB / 8;     // aux bytes per lane (CPL * AB is a multiple of 8 here)
     static_assert(AB == 0 || (CPL * AB) % 8 == 0, "aux bits of one lane must be whole bytes");
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
-    constexpr int NT = kFastWaves * 64;
+    constexpr int NT = WV * 64;
     constexpr int kKPre = CPL >= 8 ? 3 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
@@ -283,8 +283,9 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     int per_split = (blk_lim - blk_lo + p.n_splits - 1) / p.n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
-    int per_wave = (b_end - b_begin + kFastWaves - 1) / kFastWaves;
-    per_wave = (per_wave + kSuper - 1) / kSuper * kSuper;
+    int per_wave = (b_end - b_begin + WV - 1) / WV;
+    constexpr int kWaveStep = WV == 12 ? 32 : kSuper;        // ranges of whole half-steps; 64 keeps the 8-wave split as tuned
+    per_wave = (per_wave + kWaveStep - 1) / kWaveStep * kWaveStep;
     // every super-tile starts at a multiple of 64 below T_kv <= t_cap (a multiple of 64): whole tiles are readable
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
 
@@ -688,11 +689,11 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
         const int ci = cg * 16 + cc;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kFastWaves; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
+        for (int w = 0; w < WV; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
         float l = 0.f, a = 0.f;
         if (m > -INFINITY) {
 #pragma unroll
-            for (int w = 0; w < kFastWaves; w++) {
+            for (int w = 0; w < WV; w++) {
                 const float *q = red + ((size_t)w * 16 + cc) * RS;
                 const float f = __builtin_amdgcn_exp2f((q[d_h] - m) * c);
                 l = fmaf(q[d_h + 1], f, l);
@@ -711,18 +712,18 @@ __global__ __launch_bounds__(kFastWaves * 64, 2) void attn_fast_kernel(AttnParam
     }
 }
 
-template <int CPL, int MB, int AB, int IB, int DT>
+template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
-    // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 2] floats
+    // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
     size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
-    const size_t merge = (size_t)kFastWaves * 16 * (16 * CPL + 4) * sizeof(float);
+    const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);
     if (shmem < merge) shmem = merge;
-    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true> : attn_fast_kernel<CPL, MB, AB, IB, DT, false>;
+    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, kFastWaves> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
-    launch_timed(kern, grid, dim3(kFastWaves * 64), shmem, st, tm, p);
+    launch_timed(kern, grid, dim3((flags ? kFastWaves : WV) * 64), shmem, st, tm, p);
     return hip_status(hipGetLastError());
 }
 
@@ -730,8 +731,13 @@ template <int CPL, int DT>
 static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
     *handled = true;
-    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
-    if (mb == 16 && p.aux_bits == 0) return launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st, tm);
+    // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 12 % faster; the
+    // variants with more registers (other code widths, outlier caches) and short launches stay at eight
+    const bool wide = CPL == 8 && !flags && p.Tkv / p.n_splits >= 6144;
+    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12)
+        return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
+    if (mb == 16 && p.aux_bits == 0)
+        return wide ? launch_one<CPL, 16, 0, 0, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st, tm);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st, tm);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);

@@ -444,3 +444,31 @@ def test_batch_order_is_scheduling_only():
         for order in (lf, torch.tensor([4, 2, 0, 5, 3, 1], dtype=torch.int32, device=DEV)):
             O = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=2, force_generic=generic, batch_order=order)
             assert torch.equal(O, base)
+
+
+@pytest.mark.parametrize("dn,kv_lens", [("fp16", None), ("bf16", [13000, 6200])])
+def test_long_ranges_per_block(dn, kv_lens):
+    """Plain s96_r4 caches with more than 6144 tokens per block run with twelve wavefronts per block (ranges of whole
+    32-token half-steps, a merge over twelve partials): against the layout-generic kernel and dense attention."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = DT[dn]
+    B, Hq, Hkv, T, d_h = 2, 8, 2, 13000, 128
+    g = torch.Generator().manual_seed(51)
+    k, v = torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV)
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV)
+    cache = q.new_cache(B, T, d_h, dt, 0)
+    q.append(cache, k, v, 0)
+    lens = None if kv_lens is None else torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
+    Q = (torch.randn(B, Hq, 1, d_h, generator=g) * 2.0).to(dt).to(DEV)          # a peaked softmax: the merge weights matter
+    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    if lens is not None:
+        s = s.masked_fill(torch.arange(T, device=DEV).view(1, 1, 1, T) >= lens.view(B, 1, 1, 1), float("-inf"))
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
+    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))
+    for ns in (1, 2):
+        O = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns)
+        Og = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns, force_generic=True)
+        assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
