@@ -716,14 +716,15 @@ template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
     size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
-    const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);
+    const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);     // WV >= the wavefronts actually launched
     if (shmem < merge) shmem = merge;
-    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, kFastWaves> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV>;
+    constexpr int WF = CPL == 4 ? WV : kFastWaves;      // outlier variants fit three wavefronts per SIMD only at d_h 64
+    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, WF> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
-    launch_timed(kern, grid, dim3((flags ? kFastWaves : WV) * 64), shmem, st, tm, p);
+    launch_timed(kern, grid, dim3((flags ? WF : WV) * 64), shmem, st, tm, p);
     return hip_status(hipGetLastError());
 }
 
@@ -733,7 +734,7 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     *handled = true;
     // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 12 % faster; the
     // variants with more registers (other code widths, outlier caches) and short launches stay at eight
-    const bool wide = CPL == 8 && !flags && p.Tkv / p.n_splits >= 6144;
+    const bool wide = (CPL == 8 ? !flags : flags) && p.Tkv / p.n_splits >= 6144;
     if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12)
         return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 0)

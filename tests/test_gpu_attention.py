@@ -472,3 +472,27 @@ def test_long_ranges_per_block(dn, kv_lens):
         O = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns)
         Og = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns, force_generic=True)
         assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
+
+
+def test_long_ranges_per_block_outliers_d64():
+    """The d_h 64 outlier variant also runs twelve wavefronts per block above 6144 tokens per block."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.bfloat16
+    B, Hq, Hkv, T, d_h = 2, 16, 2, 13000, 64
+    k, v = _planted(B, Hkv, T, d_h, 61, dt), _planted(B, Hkv, T, d_h, 62, dt)
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV), C=3.0)
+    cache = w.new_cache(B, T, d_h, dt, 0, sideband_frac=0.25)
+    w.append(cache, k, v, 0)
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    Q = torch.randn(B, Hq, 1, d_h, generator=torch.Generator().manual_seed(63)).to(dt).to(DEV)
+    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
+    tol = 8e-3 * max(1.0, float(ref.abs().max()))
+    for ns in (1, 2):
+        O = hqmq.fused_attention_packed(Q, cache, n_splits=ns)
+        Og = hqmq.fused_attention_packed(Q, cache, n_splits=ns, force_generic=True)
+        assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
