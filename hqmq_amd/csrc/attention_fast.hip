@@ -732,15 +732,17 @@ template <int CPL, int DT>
 static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
     *handled = true;
-    // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 12 % faster; the
-    // variants with more registers (other code widths, outlier caches) and short launches stay at eight
+    // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 3-12 % faster; the
+    // variants that need more than 168 registers and short launches stay at eight
     const bool wide = (CPL == 8 ? !flags : flags) && p.Tkv / p.n_splits >= 6144;
     if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12)
         return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 0)
         return wide ? launch_one<CPL, 16, 0, 0, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st, tm);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) return launch_one<8, 12, 1, 10, DT>(p, flags, grid, st, tm);
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024)
+        return wide ? launch_one<8, 12, 1, 10, DT, 12>(p, flags, grid, st, tm) : launch_one<8, 12, 1, 10, DT>(p, flags, grid, st, tm);
     if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st, tm);
+    // (the 16+3 decode needs 182 registers: at three wavefronts per SIMD it spills and runs 40 % slower)
     if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st, tm);
     *handled = false;

@@ -446,17 +446,17 @@ def test_batch_order_is_scheduling_only():
             assert torch.equal(O, base)
 
 
-@pytest.mark.parametrize("dn,kv_lens", [("fp16", None), ("bf16", [13000, 6200])])
-def test_long_ranges_per_block(dn, kv_lens):
-    """Plain s96_r4 caches with more than 6144 tokens per block run with twelve wavefronts per block (ranges of whole
-    32-token half-steps, a merge over twelve partials): against the layout-generic kernel and dense attention."""
+@pytest.mark.parametrize("dn,kv_lens,S,b_r", [("fp16", None, 96, 4), ("bf16", [13000, 6200], 96, 4), ("bf16", None, 24, 3)])
+def test_long_ranges_per_block(dn, kv_lens, S, b_r):
+    """Plain s96_r4 and s24_r3 caches with more than 6144 tokens per block run with twelve wavefronts per block (ranges
+    of whole 32-token half-steps, a merge over twelve partials): against the layout-generic kernel and dense attention."""
     import hqmq
     from hqmq_amd import ops
     dt = DT[dn]
     B, Hq, Hkv, T, d_h = 2, 8, 2, 13000, 128
     g = torch.Generator().manual_seed(51)
     k, v = torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV)
-    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV)
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV)
     cache = q.new_cache(B, T, d_h, dt, 0)
     q.append(cache, k, v, 0)
     lens = None if kv_lens is None else torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
