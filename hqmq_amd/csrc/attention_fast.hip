@@ -236,8 +236,11 @@ __device__ __forceinline__ half4 pack4(float4v t) {
     return __builtin_bit_cast(half4, uint2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)});
 }
 
-template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS, int WV = kFastWaves>
+// NCG: column groups (of 16 columns) per wavefront.  Two for chunked prefill with more than 16 columns per KV head:
+// a decoded tile and its V transposition then serve 32 columns.
+template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS, int WV = kFastWaves, int NCG = 1>
 __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(AttnParams p) {
+    static_assert(NCG == 1 || !FLAGS, "outlier variants take one column group");
     constexpr int NB = CPL * MB / 8;
     constexpr int NW = (NB + 3) / 4;
     constexpr int ABYTES = CPL * AB / 8;     // aux bytes per lane (CPL * AB is a multiple of 8 here)
@@ -254,23 +257,29 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     const int slot = blockIdx.z / p.Hkv, hkv = blockIdx.z - slot * p.Hkv;
     const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
     const int bh = b * p.Hkv + hkv;
-    const int cg = blockIdx.y, sp = blockIdx.x;
+    const int cg0 = blockIdx.y * NCG, sp = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int G = p.G;
     constexpr int n = 4 * CPL, d_h = 16 * CPL;
     const int col = lane & 15, grp = lane >> 4;
-    const int cidx = cg * 16 + col;
-    const bool col_ok = cidx < p.Tq * G;
-    const int tq = col_ok ? cidx / G : 0, g = col_ok ? cidx - tq * G : 0;
-    const int hq = hkv * G + g;
-
     int kv_end = p.kv_len ? p.kv_len[b] : p.Tkv;
     kv_end = min(max(kv_end, 0), p.Tkv);
-    int64_t lim64 = kv_end;
-    if (p.causal) lim64 = min(lim64, (int64_t)tq + p.causal_offset + 1);
-    if (!col_ok || lim64 < 0) lim64 = 0;
-    const int col_lim = (int)lim64;
-    int blk_lim = col_lim, lim_min = col_ok ? col_lim : 0x7fffffff;
+    bool col_ok[NCG];
+    int tq[NCG], hq[NCG], col_lim[NCG];
+    int blk_lim = 0, lim_min = 0x7fffffff;
+#pragma unroll
+    for (int cgi = 0; cgi < NCG; cgi++) {
+        const int cidx = (cg0 + cgi) * 16 + col;
+        col_ok[cgi] = cidx < p.Tq * G;
+        tq[cgi] = col_ok[cgi] ? cidx / G : 0;
+        hq[cgi] = hkv * G + (col_ok[cgi] ? cidx - tq[cgi] * G : 0);
+        int64_t lim64 = kv_end;
+        if (p.causal) lim64 = min(lim64, (int64_t)tq[cgi] + p.causal_offset + 1);
+        if (!col_ok[cgi] || lim64 < 0) lim64 = 0;
+        col_lim[cgi] = (int)lim64;
+        blk_lim = max(blk_lim, col_lim[cgi]);
+        if (col_ok[cgi]) lim_min = min(lim_min, col_lim[cgi]);
+    }
     for (int o = 1; o < 16; o <<= 1) {
         blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
         lim_min = min(lim_min, __shfl_xor(lim_min, o));
@@ -334,15 +343,16 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     };
 
-    half8 qf[CPL / 2];
-    {
-        const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq * p.qsh + (int64_t)tq * p.qst + grp * CPL * 4;
+    half8 qf[NCG][CPL / 2];
+#pragma unroll
+    for (int cgi = 0; cgi < NCG; cgi++) {
+        const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[cgi] * p.qsh + (int64_t)tq[cgi] * p.qst + grp * CPL * 4;
 #pragma unroll
         for (int j = 0; j < CPL / 2; j++) {
             const half4 z = half4{0, 0, 0, 0};
-            const half4 lo = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
-            const half4 hi = col_ok ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
-            qf[j] = cat8(lo, hi);
+            const half4 lo = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
+            const half4 hi = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
+            qf[cgi][j] = cat8(lo, hi);
         }
     }
     auto load_flags = [&](int th, FlagTile &f) {
@@ -411,7 +421,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
         for (int jj = 0; jj < CPL / 2; jj++) {
-            const uint4v q8 = __builtin_bit_cast(uint4v, qf[jj]);
+            const uint4v q8 = __builtin_bit_cast(uint4v, qf[0][jj]);
             const int c0 = grp * CPL + 2 * jj;
             lds_tab[kQOffset / 8 + c0 * 16 + col] = uint2{q8[0], q8[1]};
             lds_tab[kQOffset / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
@@ -437,10 +447,15 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 
     // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
     const float c = p.c_log2, qmaxf = (float)p.qmax;
-    float m_run = -INFINITY, l_run = 0.f;
-    float4v acc[CPL];
+    float m_run[NCG], l_run[NCG];
+    float4v acc[NCG][CPL];
 #pragma unroll
-    for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int cgi = 0; cgi < NCG; cgi++) {
+        m_run[cgi] = -INFINITY;
+        l_run[cgi] = 0.f;
+#pragma unroll
+        for (int j = 0; j < CPL; j++) acc[cgi][j] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
     const half4 zero_h4 = half4{0, 0, 0, 0};
     // Every load of the loop is issued unconditionally (clamped addresses): a load inside a branch would make the
@@ -526,7 +541,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             const bool mj = owner && jq == j;
             if (__builtin_amdgcn_ballot_w64(mj) != 0) {
                 const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
             }
         }
     };
@@ -546,69 +561,80 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // carries radius code 0 in the main plane, so its decoded value is exactly zero and only the verbatim
     // value from the sideband contributes.
     auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre<kKPre> &kc, const VPre<kVPre> &vc) {
-        float4v sT[2], so[2] = {zero4, zero4};
+        float4v sT[NCG][2], so[2] = {zero4, zero4};
         if (FLAGS) k_apply(kc, so);
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
             decode_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, a);
-            float4v s = zero4;
 #pragma unroll
-            for (int jj = 0; jj < CPL / 2; jj++)
-                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
+            for (int cgi = 0; cgi < NCG; cgi++) {
+                float4v s = zero4;
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[u][e] * qmaxf : 0.f);
-            sT[u] = s;
+                for (int jj = 0; jj < CPL / 2; jj++)
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[cgi][jj], s, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[u][e] * qmaxf : 0.f);
+                sT[cgi][u] = s;
+            }
         }
-        // ---- mask (boundary half-steps only), online softmax ----
-        if (!(th + 32 <= lim_min && th + 32 <= t_end && th >= col_start)) {
+        // ---- mask (boundary half-steps only), online softmax, per column group ----
+        const bool edge = !(th + 32 <= lim_min && th + 32 <= t_end && th >= col_start);
+        half8 pp[NCG];
+        half4 pTo[2];
 #pragma unroll
-            for (int u = 0; u < 2; u++)
+        for (int cgi = 0; cgi < NCG; cgi++) {
+            if (edge) {
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int t = th + 16 * u + 4 * grp + e;
+                        if (!(t < col_lim[cgi] && t < t_end && t >= col_start)) sT[cgi][u][e] = -INFINITY;
+                    }
+            }
+            float tmax = fmaxf(fmaxf(fmaxf(sT[cgi][0][0], sT[cgi][0][1]), fmaxf(sT[cgi][0][2], sT[cgi][0][3])),
+                               fmaxf(fmaxf(sT[cgi][1][0], sT[cgi][1][1]), fmaxf(sT[cgi][1][2], sT[cgi][1][3])));
+            tmax = row_max4(tmax);
+            const float m_new = fmaxf(m_run[cgi], tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            if (__builtin_amdgcn_ballot_w64(m_new != m_run[cgi]) != 0) {     // rescale only when some column's maximum moved
+                const float alpha = __builtin_amdgcn_exp2f((m_run[cgi] - m_use) * c);
+                l_run[cgi] *= alpha;
+#pragma unroll
+                for (int j = 0; j < CPL; j++) acc[cgi][j] = acc[cgi][j] * alpha;
+                m_run[cgi] = m_new;
+            }
+            const float mc = -m_use * c;
+            half4 pT[2];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                float pe[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const int t = th + 16 * u + 4 * grp + e;
-                    if (!(t < col_lim && t < t_end && t >= col_start)) sT[u][e] = -INFINITY;
+                    pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[cgi][u][e], c, mc));
+                    l_run[cgi] += pe[e];
                 }
-        }
-        float tmax = fmaxf(fmaxf(fmaxf(sT[0][0], sT[0][1]), fmaxf(sT[0][2], sT[0][3])),
-                           fmaxf(fmaxf(sT[1][0], sT[1][1]), fmaxf(sT[1][2], sT[1][3])));
-        tmax = row_max4(tmax);
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {     // rescale only when some column's maximum moved
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-            l_run *= alpha;
-#pragma unroll
-            for (int j = 0; j < CPL; j++) acc[j] = acc[j] * alpha;
-            m_run = m_new;
-        }
-        const float mc = -m_use * c;
-        half4 pT[2], pTo[2];
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            float pe[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[u][e], c, mc));
-                l_run += pe[e];
+                const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(h.vs[u].x);
+                const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(h.vs[u].y);
+                pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
+                if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
             }
-            const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(h.vs[u].x);
-            const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(h.vs[u].y);
-            pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
-            if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
+            pp[cgi] = cat8(pT[0], pT[1]);
         }
         // ---- O^T += V^T . P^T, both tiles in one MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
         half4 av[2][CPL];
 #pragma unroll
         for (int u = 0; u < 2; u++)
             decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, av[u]);
-        const half8 pp = cat8(pT[0], pT[1]);
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
             const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
+            const half8 vt = cat8(pack4(t0v), pack4(t1v));
+#pragma unroll
+            for (int cgi = 0; cgi < NCG; cgi++) acc[cgi][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pp[cgi], acc[cgi][j], 0, 0, 0);
         }
         if (FLAGS) v_apply(vc, cat8(pTo[0], pTo[1]));
     };
@@ -670,56 +696,61 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     }
 
-    // ---- merge the block's waves through LDS: rows of [d_h accumulators, m, l, pad] ----
+    // ---- merge the block's waves through LDS: rows of [d_h accumulators, m, l, pad], one column group at a time ----
     constexpr int RS = d_h + 4;
-    const float l_tot = row_sum4(l_run);
     float *red = reinterpret_cast<float *>(lds_tab);            // [wave][16 cols][RS]
-    __syncthreads();
-    const int ncols = min(16, p.Tq * G - cg * 16);
-    if (col < ncols) {                                          // padding columns are never read back
-        float *wp = red + ((size_t)wave * 16 + col) * RS;
-        if (grp == 0) { wp[d_h] = m_run; wp[d_h + 1] = l_tot; }
-#pragma unroll
-        for (int j = 0; j < CPL; j++) *reinterpret_cast<float4v *>(wp + grp * CPL * 4 + 4 * j) = acc[j];
-    }
-    __syncthreads();
     const float inv_qmax = p.inv_qmax;
-    for (int o = threadIdx.x; o < ncols * d_h; o += NT) {
-        const int cc = o / d_h, e = o - cc * d_h;
-        const int ci = cg * 16 + cc;
-        float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WV; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
-        float l = 0.f, a = 0.f;
-        if (m > -INFINITY) {
+    for (int cgi = 0; cgi < NCG; cgi++) {
+        const int cg = cg0 + cgi;
+        const float l_tot = row_sum4(l_run[cgi]);
+        __syncthreads();
+        const int ncols = min(16, p.Tq * G - cg * 16);          // <= 0 for a column group past the end
+        if (col < ncols) {                                      // padding columns are never read back
+            float *wp = red + ((size_t)wave * 16 + col) * RS;
+            if (grp == 0) { wp[d_h] = m_run[cgi]; wp[d_h + 1] = l_tot; }
 #pragma unroll
-            for (int w = 0; w < WV; w++) {
-                const float *q = red + ((size_t)w * 16 + cc) * RS;
-                const float f = __builtin_amdgcn_exp2f((q[d_h] - m) * c);
-                l = fmaf(q[d_h + 1], f, l);
-                a = fmaf(q[e], f, a);
-            }
+            for (int j = 0; j < CPL; j++) *reinterpret_cast<float4v *>(wp + grp * CPL * 4 + 4 * j) = acc[cgi][j];
         }
-        const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
-        if (p.n_splits == 1) {
-            store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
-        } else {
-            // partials carry the maximum in softmax units (base-2 exponent) and acc already divided by qmax
-            float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
-            if (e == 0) { wp[0] = m * c; wp[1] = l; }
-            wp[2 + e] = a * inv_qmax;
+        __syncthreads();
+        for (int o = threadIdx.x; o < ncols * d_h; o += NT) {
+            const int cc = o / d_h, e = o - cc * d_h;
+            const int ci = cg * 16 + cc;
+            float m = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < WV; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
+            float l = 0.f, a = 0.f;
+            if (m > -INFINITY) {
+#pragma unroll
+                for (int w = 0; w < WV; w++) {
+                    const float *q = red + ((size_t)w * 16 + cc) * RS;
+                    const float f = __builtin_amdgcn_exp2f((q[d_h] - m) * c);
+                    l = fmaf(q[d_h + 1], f, l);
+                    a = fmaf(q[e], f, a);
+                }
+            }
+            const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
+            if (p.n_splits == 1) {
+                store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
+            } else {
+                // partials carry the maximum in softmax units (base-2 exponent) and acc already divided by qmax
+                float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
+                if (e == 0) { wp[0] = m * c; wp[1] = l; }
+                wp[2 + e] = a * inv_qmax;
+            }
         }
     }
 }
 
-template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves>
+template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves, int NCG = 1>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
+    if (NCG > 1) grid.y = (grid.y + NCG - 1) / NCG;
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
     size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);     // WV >= the wavefronts actually launched
     if (shmem < merge) shmem = merge;
     constexpr int WF = CPL == 4 ? WV : kFastWaves;      // outlier variants fit three wavefronts per SIMD only at d_h 64
-    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, WF> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV>;
+    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, WF> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV, NCG>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
@@ -735,15 +766,25 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 3-12 % faster; the
     // variants that need more than 168 registers and short launches stay at eight
     const bool wide = (CPL == 8 ? !flags : flags) && p.Tkv / p.n_splits >= 6144;
-    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12)
+    // chunked prefill (more than 16 columns per KV head) of plain caches: two column groups per wavefront
+    // (only while a block per CU is left: fewer, larger blocks lose more than the shared decode wins)
+    const bool two = !flags && p.n_cg > 1 && (int64_t)p.n_splits * ((p.n_cg + 1) / 2) * p.B * p.Hkv >= 256;
+    if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) {
+        if (two) return launch_one<CPL, 16, 0, 12, DT, kFastWaves, 2>(p, flags, grid, st, tm);
         return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
-    if (mb == 16 && p.aux_bits == 0)
+    }
+    if (mb == 16 && p.aux_bits == 0) {
+        if (two) return launch_one<CPL, 16, 0, 0, DT, kFastWaves, 2>(p, flags, grid, st, tm);
         return wide ? launch_one<CPL, 16, 0, 0, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 0, DT>(p, flags, grid, st, tm);
-    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024)
+    }
+    if (mb == 12 && p.aux_bits == 1 && CPL == 8 && p.idx_bits == 10 && p.Kc.K <= 1024) {
+        if (two) return launch_one<8, 12, 1, 10, DT, kFastWaves, 2>(p, flags, grid, st, tm);
         return wide ? launch_one<8, 12, 1, 10, DT, 12>(p, flags, grid, st, tm) : launch_one<8, 12, 1, 10, DT>(p, flags, grid, st, tm);
+    }
     if (mb == 12 && p.aux_bits == 1 && CPL == 8) return launch_one<8, 12, 1, 0, DT>(p, flags, grid, st, tm);
     // (the 16+3 decode needs 182 registers: at three wavefronts per SIMD it spills and runs 40 % slower)
-    if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);
+    if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608)
+        return two ? launch_one<8, 16, 3, 13, DT, kFastWaves, 2>(p, flags, grid, st, tm) : launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st, tm);
     *handled = false;
     return HQMQ_OK;

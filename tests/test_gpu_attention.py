@@ -496,3 +496,32 @@ def test_long_ranges_per_block_outliers_d64():
         O = hqmq.fused_attention_packed(Q, cache, n_splits=ns)
         Og = hqmq.fused_attention_packed(Q, cache, n_splits=ns, force_generic=True)
         assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
+
+
+@pytest.mark.parametrize("S,b_r,dn,d_h", [(96, 4, "fp16", 128), (24, 3, "bf16", 128), (192, 6, "fp16", 128), (96, 4, "bf16", 64)])
+def test_prefill_two_column_groups(S, b_r, dn, d_h):
+    """Chunked prefill with enough columns for a block per CU runs two column groups per wavefront on plain caches
+    (an odd number of groups, a last group that is partly padding, causal limits that differ inside a wavefront):
+    against dense attention and the layout-generic kernel."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = DT[dn]
+    B, Hq, Hkv, T, Tq = 2, 8, 2, 700, 299
+    g = torch.Generator().manual_seed(71)
+    k, v = torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV)
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV)
+    cache = q.new_cache(B, T, d_h, dt, 0)
+    q.append(cache, k, v, 0)
+    Q = torch.randn(B, Hq, Tq, d_h, generator=g).to(dt).to(DEV)
+    off = T - Tq
+    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
+    mask = torch.arange(T, device=DEV).view(1, 1, 1, T) <= (torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off)
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
+    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))
+    for ns in (2, 4):                       # 2 splits x 38 pairs of column groups x 4 (b, h) = 304 blocks
+        O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=ns)
+        assert (O.float() - ref).abs().max().item() < tol, ns
+    Og = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=2, force_generic=True)
+    assert (Og.float() - ref).abs().max().item() < tol
