@@ -525,3 +525,11 @@ def test_prefill_two_column_groups(S, b_r, dn, d_h):
         assert (O.float() - ref).abs().max().item() < tol, ns
     Og = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=2, force_generic=True)
     assert (Og.float() - ref).abs().max().item() < tol
+    # the same with per-sequence limits on both sides (left padding and a shorter second sequence)
+    starts = torch.tensor([0, 70], dtype=torch.int32, device=DEV)
+    lens = torch.tensor([T, 650], dtype=torch.int32, device=DEV)
+    kk = torch.arange(T, device=DEV).view(1, 1, 1, T)
+    mask2 = mask & (kk >= starts.view(B, 1, 1, 1)) & (kk < lens.view(B, 1, 1, 1))
+    ref2 = torch.einsum("bhqk,bhkd->bhqd", torch.nan_to_num(torch.softmax(s.masked_fill(~mask2, float("-inf")), -1)), Vd)
+    O2 = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=2, kv_starts=starts, kv_lens=lens, T_kv=T)
+    assert (O2.float() - ref2).abs().max().item() < tol
