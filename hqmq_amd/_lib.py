@@ -38,6 +38,15 @@ class QuantizeArgs(C.Structure):
     ]
 
 
+class AppendArgs(C.Structure):
+    _fields_ = [
+        ("q", QuantizeArgs), ("median_mult", C.c_float),
+        ("med_workspace", vp), ("med_workspace_bytes", i64),
+        ("median", vp), ("thr", vp), ("n_out", vp),
+        ("sideband", vp), ("sb_cap", i64), ("sb_tile_off", vp), ("sb_count", vp), ("overflow", vp), ("sb_coord", vp),
+    ]
+
+
 class Packed(C.Structure):
     _fields_ = [
         ("main_plane", vp), ("aux_plane", vp), ("flag_plane", vp), ("scale_plane", vp),
@@ -65,7 +74,7 @@ EXPORTS = [
     "hqmq_version", "hqmq_status_string", "hqmq_layout_bits", "hqmq_build_joint", "hqmq_quantize",
     "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",
     "hqmq_pack_codes", "hqmq_dequant_packed", "hqmq_attn_workspace_bytes", "hqmq_attn_pick_splits",
-    "hqmq_attn_fwd", "hqmq_attn_combine",
+    "hqmq_attn_fwd", "hqmq_attn_combine", "hqmq_append_kv",
 ]
 
 

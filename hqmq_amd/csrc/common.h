@@ -86,4 +86,24 @@ inline int layout_bits(int S, int radius_bits, int *idx_bits, int *main_bits, in
 
 inline int hip_status(hipError_t e) { return e == hipSuccess ? HQMQ_OK : (int)e; }
 
+// ---- the stages of an append, for one tensor or for the K and the V tensor of a cache together ----
+// With two calls of equal shape every stage is one launch whose blocks split between the tensors; otherwise the
+// calls run one after the other.  Results are those of the single-tensor entry points either way.
+struct Med3xCall {
+    const void *x; int64_t xsb, xsh, xst;
+    int dtype, B, H, T, n;
+    float mult;
+    void *ws; int64_t ws_bytes;
+    float *median; void *thr; int32_t *n_out;
+};
+struct CompactCall {
+    const void *x; int64_t xsb, xsh, xst;
+    int dtype, B, H, T, n;
+    const uint8_t *flag_plane; int64_t t_cap; int t_off; const int32_t *pos;
+    void *sideband; int64_t sb_cap; int32_t *sb_tile_off, *sb_count, *overflow; uint16_t *sb_coord;
+};
+int med3x_calls(const Med3xCall *c, int count, hipStream_t st);                                            // med3x.hip
+int compact_calls(const CompactCall *c, int count, hipStream_t st);                                        // med3x.hip
+int quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, hipStream_t st);                // quantize.hip
+
 }  // namespace hqmq

@@ -243,10 +243,22 @@ __device__ __forceinline__ void find_bin256(const uint32_t *hist, uint32_t rank,
     __syncthreads();
 }
 
+struct MedSmall {
+    const void *x; int64_t xsb, xsh, xst;
+    int B, T, n;
+    float mult;
+    float *median; void *thr; int32_t *n_out;
+};
+
 template <class D>
-__global__ __launch_bounds__(1024) void med_small_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int B,
-                                                         int T, int n, float mult, float *median, typename D::storage *thr,
-                                                         int32_t *n_out) {
+__device__ __forceinline__ void med_small_body(const MedSmall &a) {
+    const typename D::storage *x = (const typename D::storage *)a.x;
+    typename D::storage *thr = (typename D::storage *)a.thr;
+    const int64_t xsb = a.xsb, xsh = a.xsh, xst = a.xst;
+    const int B = a.B, T = a.T, n = a.n;
+    const float mult = a.mult;
+    float *median = a.median;
+    int32_t *n_out = a.n_out;
     __shared__ uint16_t keys[kSmallMax];
     __shared__ uint32_t hist[256], wave_tot[4], res[2], nan_count, gt_count;
     __shared__ float thr_sh;
@@ -308,6 +320,16 @@ __global__ __launch_bounds__(1024) void med_small_kernel(const typename D::stora
     }
 }
 
+template <class D>
+__global__ __launch_bounds__(1024) void med_small_kernel(MedSmall a) {
+    med_small_body<D>(a);
+}
+// two tensors of equal shape: blockIdx.y picks one
+template <class D>
+__global__ __launch_bounds__(1024) void med_small_pair_kernel(MedSmall a, MedSmall b) {
+    med_small_body<D>(blockIdx.y ? b : a);
+}
+
 __global__ __launch_bounds__(1024) void med_select2_kernel(uint32_t *ws, int H, int64_t per_head, float mult, float *median,
                                                            float *thr) {
     const int h = blockIdx.x;
@@ -346,11 +368,16 @@ __global__ void count_gt_kernel(const float *x, int64_t xsb, int64_t xsh, int64_
 
 // One block per (b, h): walks the T new rows in order, 1024 rows per step.
 template <class D>
-__global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H,
-                                                        int T, int n, const uint8_t *flag_plane, int64_t t_cap, int t_off,
-                                                        const int32_t *pos, typename D::storage *sideband, int64_t sb_cap,
-                                                        int32_t *sb_tile_off, int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord) {
+__device__ __forceinline__ void compact_body(const CompactCall &a) {
     using ST = typename D::storage;
+    const ST *x = (const ST *)a.x;
+    ST *sideband = (ST *)a.sideband;
+    const int64_t xsb = a.xsb, xsh = a.xsh, xst = a.xst, t_cap = a.t_cap, sb_cap = a.sb_cap;
+    const int H = a.H, T = a.T, n = a.n, t_off = a.t_off;
+    const uint8_t *flag_plane = a.flag_plane;
+    const int32_t *pos = a.pos;
+    int32_t *sb_tile_off = a.sb_tile_off, *sb_count = a.sb_count, *overflow = a.overflow;
+    uint16_t *sb_coord = a.sb_coord;
     __shared__ int scan[1024];
     __shared__ int base_sh;
     const int bh = blockIdx.x, b = bh / H, h = bh - b * H;
@@ -397,6 +424,16 @@ __global__ __launch_bounds__(1024) void compact_kernel(const typename D::storage
         __syncthreads();
     }
     if (threadIdx.x == 0) sb_count[bh] = base_sh;
+}
+
+template <class D>
+__global__ __launch_bounds__(1024) void compact_kernel(CompactCall a) {
+    compact_body<D>(a);
+}
+// two tensors of equal shape: blockIdx.y picks one
+template <class D>
+__global__ __launch_bounds__(1024) void compact_pair_kernel(CompactCall a, CompactCall b) {
+    compact_body<D>(blockIdx.y ? b : a);
 }
 
 // ---- bulk appends (whole 16-row tiles from an aligned first row): three passes with one thread per tile / row ----
@@ -490,8 +527,7 @@ static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B
     const int64_t words = ws_words(H, f32);
     const int64_t per_head = (int64_t)B * T * n;
     if (!f32 && per_head <= kSmallMax) {
-        hipLaunchKernelGGL(med_small_kernel<D>, dim3(H), dim3(1024), 0, st, (const ST *)x, xsb, xsh, xst, B, T, n, mult, median,
-                           (ST *)thr, n_out);
+        hipLaunchKernelGGL(med_small_kernel<D>, dim3(H), dim3(1024), 0, st, MedSmall{x, xsb, xsh, xst, B, T, n, mult, median, thr, n_out});
         return hip_status(hipGetLastError());
     }
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, ws, words);
@@ -520,61 +556,121 @@ static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B
     return hip_status(hipGetLastError());
 }
 
+static int check_med3x(const Med3xCall &c) {
+    if (!c.x || !c.ws || !c.median || !c.thr) return HQMQ_ERR_NULL;
+    if (c.B < 1 || c.H < 1 || c.H > 65535 || c.T < 1 || c.n < 1) return HQMQ_ERR_SHAPE;
+    if (c.dtype != HQMQ_F32 && c.dtype != HQMQ_F16 && c.dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
+    if (c.ws_bytes < hqmq_med3x_workspace_bytes(c.H, c.dtype)) return HQMQ_ERR_WORKSPACE;
+    if (((uintptr_t)c.ws & 3) != 0) return HQMQ_ERR_ALIGN;
+    return HQMQ_OK;
+}
+
+static int med3x_one(const Med3xCall &c, hipStream_t st) {
+    uint32_t *ws = (uint32_t *)c.ws;
+    switch (c.dtype) {
+        case HQMQ_F32: return run_med3x<F32>(c.x, c.xsb, c.xsh, c.xst, c.B, c.H, c.T, c.n, c.mult, ws, c.median, c.thr, c.n_out, st);
+        case HQMQ_F16: return run_med3x<F16>(c.x, c.xsb, c.xsh, c.xst, c.B, c.H, c.T, c.n, c.mult, ws, c.median, c.thr, c.n_out, st);
+        default: return run_med3x<BF16>(c.x, c.xsb, c.xsh, c.xst, c.B, c.H, c.T, c.n, c.mult, ws, c.median, c.thr, c.n_out, st);
+    }
+}
+
+int hqmq::med3x_calls(const Med3xCall *c, int count, hipStream_t st) {
+    for (int i = 0; i < count; i++) {
+        const int rc = check_med3x(c[i]);
+        if (rc) return rc;
+    }
+    if (count == 2 && c[0].dtype == c[1].dtype && c[0].dtype != HQMQ_F32 && c[0].B == c[1].B && c[0].H == c[1].H &&
+        c[0].T == c[1].T && c[0].n == c[1].n && (int64_t)c[0].B * c[0].T * c[0].n <= kSmallMax) {
+        const MedSmall a{c[0].x, c[0].xsb, c[0].xsh, c[0].xst, c[0].B, c[0].T, c[0].n, c[0].mult, c[0].median, c[0].thr, c[0].n_out};
+        const MedSmall b{c[1].x, c[1].xsb, c[1].xsh, c[1].xst, c[1].B, c[1].T, c[1].n, c[1].mult, c[1].median, c[1].thr, c[1].n_out};
+        if (c[0].dtype == HQMQ_F16) hipLaunchKernelGGL(med_small_pair_kernel<F16>, dim3(c[0].H, 2), dim3(1024), 0, st, a, b);
+        else hipLaunchKernelGGL(med_small_pair_kernel<BF16>, dim3(c[0].H, 2), dim3(1024), 0, st, a, b);
+        return hip_status(hipGetLastError());
+    }
+    for (int i = 0; i < count; i++) {
+        const int rc = med3x_one(c[i], st);
+        if (rc) return rc;
+    }
+    return HQMQ_OK;
+}
+
 extern "C" int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
                                     int H, int T, int n_chunks, float mult, void *workspace, int64_t workspace_bytes,
                                     float *median, void *thr, int32_t *n_out, void *stream) {
-    if (!x || !workspace || !median || !thr) return HQMQ_ERR_NULL;
-    if (B < 1 || H < 1 || H > 65535 || T < 1 || n_chunks < 1) return HQMQ_ERR_SHAPE;
-    if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
-    if (workspace_bytes < hqmq_med3x_workspace_bytes(H, dtype)) return HQMQ_ERR_WORKSPACE;
-    if (((uintptr_t)workspace & 3) != 0) return HQMQ_ERR_ALIGN;
-    hipStream_t st = (hipStream_t)stream;
-    uint32_t *ws = (uint32_t *)workspace;
-    switch (dtype) {
-        case HQMQ_F32: return run_med3x<F32>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
-        case HQMQ_F16: return run_med3x<F16>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
-        default: return run_med3x<BF16>(x, x_stride_b, x_stride_h, x_stride_t, B, H, T, n_chunks, mult, ws, median, thr, n_out, st);
+    const Med3xCall c{x, x_stride_b, x_stride_h, x_stride_t, dtype, B, H, T, n_chunks, mult, workspace, workspace_bytes,
+                      median, thr, n_out};
+    return med3x_calls(&c, 1, (hipStream_t)stream);
+}
+
+static int check_compact(const CompactCall &c) {
+    if (!c.x || !c.flag_plane || !c.sideband || !c.sb_tile_off || !c.sb_count || !c.overflow) return HQMQ_ERR_NULL;
+    if (c.B < 1 || c.H < 1 || c.T < 0 || c.n < 1 || c.t_cap < 1 || c.sb_cap < 1 || c.t_off < 0) return HQMQ_ERR_SHAPE;
+    if (c.dtype != HQMQ_F32 && c.dtype != HQMQ_F16 && c.dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
+    return HQMQ_OK;
+}
+
+// whole 16-row tiles from an aligned first row: the three tile-parallel passes
+static bool bulk_compact(const CompactCall &c) {
+    return !c.pos && (c.t_off % kTile) == 0 && c.T >= 512 && (int64_t)c.t_off + c.T <= c.t_cap && c.B * c.H <= 65535;
+}
+
+static int compact_one(const CompactCall &c, hipStream_t st) {
+    if (c.T == 0) return HQMQ_OK;
+    if (bulk_compact(c)) {
+        const int n_tiles = (c.T + kTile - 1) / kTile, frb = (c.n + 7) >> 3;
+        hipLaunchKernelGGL(tile_count_kernel, dim3((n_tiles + 255) / 256, c.B * c.H), dim3(256), 0, st, c.flag_plane, c.t_cap, c.t_off,
+                           c.T, frb, n_tiles, c.sb_tile_off);
+        hipLaunchKernelGGL(tile_scan_kernel, dim3(c.B * c.H), dim3(1024), 0, st, c.t_cap, c.t_off, n_tiles, c.sb_tile_off, c.sb_count);
+        dim3 cgrid((c.T + 255) / 256, c.B * c.H);
+#define COPY(DT, ST)                                                                                                       \
+    hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, (const ST *)c.x, c.xsb, c.xsh, c.xst, c.H, c.T, c.n,     \
+                       c.flag_plane, c.t_cap, c.t_off, (ST *)c.sideband, c.sb_cap, c.sb_tile_off, c.overflow, c.sb_coord)
+        switch (c.dtype) {
+            case HQMQ_F32: COPY(F32, float); break;
+            case HQMQ_F16: COPY(F16, uint16_t); break;
+            default: COPY(BF16, uint16_t); break;
+        }
+#undef COPY
+        return hip_status(hipGetLastError());
     }
+    dim3 grid(c.B * c.H), block(1024);
+    switch (c.dtype) {
+        case HQMQ_F32: hipLaunchKernelGGL(compact_kernel<F32>, grid, block, 0, st, c); break;
+        case HQMQ_F16: hipLaunchKernelGGL(compact_kernel<F16>, grid, block, 0, st, c); break;
+        default: hipLaunchKernelGGL(compact_kernel<BF16>, grid, block, 0, st, c); break;
+    }
+    return hip_status(hipGetLastError());
+}
+
+int hqmq::compact_calls(const CompactCall *c, int count, hipStream_t st) {
+    for (int i = 0; i < count; i++) {
+        const int rc = check_compact(c[i]);
+        if (rc) return rc;
+    }
+    if (count == 2 && c[0].T > 0 && c[0].dtype == c[1].dtype && c[0].B == c[1].B && c[0].H == c[1].H && c[0].T == c[1].T &&
+        c[0].n == c[1].n && !bulk_compact(c[0]) && !bulk_compact(c[1])) {
+        dim3 grid(c[0].B * c[0].H, 2), block(1024);
+        switch (c[0].dtype) {
+            case HQMQ_F32: hipLaunchKernelGGL(compact_pair_kernel<F32>, grid, block, 0, st, c[0], c[1]); break;
+            case HQMQ_F16: hipLaunchKernelGGL(compact_pair_kernel<F16>, grid, block, 0, st, c[0], c[1]); break;
+            default: hipLaunchKernelGGL(compact_pair_kernel<BF16>, grid, block, 0, st, c[0], c[1]); break;
+        }
+        return hip_status(hipGetLastError());
+    }
+    for (int i = 0; i < count; i++) {
+        const int rc = compact_one(c[i], st);
+        if (rc) return rc;
+    }
+    return HQMQ_OK;
 }
 
 extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
                                     int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
                                     const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off,
                                     int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord, void *stream) {
-    if (!x || !flag_plane || !sideband || !sb_tile_off || !sb_count || !overflow) return HQMQ_ERR_NULL;
-    if (B < 1 || H < 1 || T < 0 || n_chunks < 1 || t_cap < 1 || sb_cap < 1 || t_off < 0) return HQMQ_ERR_SHAPE;
-    if (T == 0) return HQMQ_OK;
-    hipStream_t st = (hipStream_t)stream;
-    if (!pos && (t_off % kTile) == 0 && T >= 512 && (int64_t)t_off + T <= t_cap && B * H <= 65535) {
-        const int n_tiles = (T + kTile - 1) / kTile, frb = (n_chunks + 7) >> 3;
-        hipLaunchKernelGGL(tile_count_kernel, dim3((n_tiles + 255) / 256, B * H), dim3(256), 0, st, flag_plane, t_cap, t_off, T, frb,
-                           n_tiles, sb_tile_off);
-        hipLaunchKernelGGL(tile_scan_kernel, dim3(B * H), dim3(1024), 0, st, t_cap, t_off, n_tiles, sb_tile_off, sb_count);
-        dim3 cgrid((T + 255) / 256, B * H);
-#define COPY(DT, ST)                                                                                                          \
-    hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T,    \
-                       n_chunks, flag_plane, t_cap, t_off, (ST *)sideband, sb_cap, sb_tile_off, overflow, sb_coord)
-        switch (dtype) {
-            case HQMQ_F32: COPY(F32, float); break;
-            case HQMQ_F16: COPY(F16, uint16_t); break;
-            case HQMQ_BF16: COPY(BF16, uint16_t); break;
-            default: return HQMQ_ERR_DTYPE;
-        }
-#undef COPY
-        return hip_status(hipGetLastError());
-    }
-    dim3 grid(B * H), block(1024);
-#define LAUNCH(DT, ST)                                                                                                      \
-    hipLaunchKernelGGL(compact_kernel<DT>, grid, block, 0, st, (const ST *)x, x_stride_b, x_stride_h, x_stride_t, H, T, n_chunks, \
-                       flag_plane, t_cap, t_off, pos, (ST *)sideband, sb_cap, sb_tile_off, sb_count, overflow, sb_coord)
-    switch (dtype) {
-        case HQMQ_F32: LAUNCH(F32, float); break;
-        case HQMQ_F16: LAUNCH(F16, uint16_t); break;
-        case HQMQ_BF16: LAUNCH(BF16, uint16_t); break;
-        default: return HQMQ_ERR_DTYPE;
-    }
-#undef LAUNCH
-    return hip_status(hipGetLastError());
+    const CompactCall c{x, x_stride_b, x_stride_h, x_stride_t, dtype, B, H, T, n_chunks, flag_plane, t_cap, t_off, pos,
+                        sideband, sb_cap, sb_tile_off, sb_count, overflow, sb_coord};
+    return compact_calls(&c, 1, (hipStream_t)stream);
 }
 
 namespace hqmq {

@@ -129,7 +129,7 @@ __device__ __forceinline__ uint8_t gather_byte(const uint32_t *vals, int count, 
 }
 
 template <class D, int ALGO>
-__global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
+__device__ __forceinline__ void quantize_body(const QParams &a) {
     using ST = typename D::storage;
     extern __shared__ float sec[];  // [S][4] secondaries, then [S][4] fp16 columns of their rotation matrices
     uint2 *rot = reinterpret_cast<uint2 *>(sec + 4 * a.S);
@@ -367,12 +367,32 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
     }
 }
 
+template <class D, int ALGO>
+__global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
+    quantize_body<D, ALGO>(a);
+}
+
+// The K and the V rows of one append in one launch (same shapes): blockIdx.z picks the tensor.  A single-token
+// append is latency-bound (32 lanes per block for a few microseconds), so the two run side by side for free.
+template <class D>
+__global__ __launch_bounds__(kQThreads) void quantize_pair_kernel(QParams k, QParams v) {
+    quantize_body<D, 0>(blockIdx.z ? v : k);
+}
+
 template <class D>
 static int launch_quantize(const QParams &p, int algo, hipStream_t st) {
     dim3 grid((p.T + p.tokens_per_block - 1) / p.tokens_per_block, p.B * p.H), block(kQThreads);
     size_t shmem = (size_t)p.S * 4 * sizeof(float) + (size_t)p.S * 4 * sizeof(uint2);
     if (algo == 1) hipLaunchKernelGGL((quantize_kernel<D, 1>), grid, block, shmem, st, p);
     else hipLaunchKernelGGL((quantize_kernel<D, 0>), grid, block, shmem, st, p);
+    return hip_status(hipGetLastError());
+}
+
+template <class D>
+static int launch_quantize_pair(const QParams &k, const QParams &v, hipStream_t st) {
+    dim3 grid((k.T + k.tokens_per_block - 1) / k.tokens_per_block, k.B * k.H, 2), block(kQThreads);
+    size_t shmem = (size_t)k.S * 4 * sizeof(float) + (size_t)k.S * 4 * sizeof(uint2);
+    hipLaunchKernelGGL(quantize_pair_kernel<D>, grid, block, shmem, st, k, v);
     return hip_status(hipGetLastError());
 }
 
@@ -384,12 +404,14 @@ extern "C" int hqmq_layout_bits(int S, int radius_bits, int *idx_bits, int *main
     return layout_bits(S, radius_bits, idx_bits, main_bits, aux_bits);
 }
 
-extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
+// Checks one call's arguments and fills the kernel parameters; *empty is set for T == 0 (nothing to launch).
+static int fill_qparams(const hqmq_quantize_args *a, QParams *out, bool *empty) {
+    *empty = false;
     if (!a || !a->x || !a->joint) return HQMQ_ERR_NULL;
     if (a->algo == 0 && !a->slack) return HQMQ_ERR_NULL;
     if (a->B < 1 || a->H < 1 || a->T < 0 || a->n_chunks < 1 || a->n_chunks > kQThreads) return HQMQ_ERR_SHAPE;
     if ((int64_t)a->B * a->H > 65535) return HQMQ_ERR_SHAPE;
-    if (a->T == 0) return HQMQ_OK;
+    if (a->T == 0) { *empty = true; return HQMQ_OK; }
     int ib, mb, ab;
     int rc = layout_bits(a->secondary_size, a->radius_bits, &ib, &mb, &ab);
     if (rc) return rc;
@@ -406,7 +428,8 @@ extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
         if (!a->pos && (int64_t)a->t_off + a->T > a->t_cap) return HQMQ_ERR_SHAPE;
         if (a->flag_plane && !a->thr) return HQMQ_ERR_NULL;
     }
-    QParams p;
+    if (a->dtype != HQMQ_F32 && a->dtype != HQMQ_F16 && a->dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
+    QParams &p = *out;
     p.x = a->x; p.xsb = a->x_stride_b; p.xsh = a->x_stride_h; p.xst = a->x_stride_t;
     p.B = a->B; p.H = a->H; p.T = a->T; p.n = a->n_chunks;
     p.joint = a->joint; p.slack = a->slack; p.S = a->secondary_size; p.qmax = (1 << a->radius_bits) - 1;
@@ -417,11 +440,44 @@ extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
     p.idx_bits = ib; p.main_bits = packed ? a->main_bits : mb; p.aux_bits = packed ? a->aux_bits : ab;
     p.tokens_per_block = kQThreads / a->n_chunks;
     p.stats = a->stats;
-    hipStream_t st = (hipStream_t)stream;
-    switch (a->dtype) {
-        case HQMQ_F32: return launch_quantize<F32>(p, a->algo, st);
-        case HQMQ_F16: return launch_quantize<F16>(p, a->algo, st);
-        case HQMQ_BF16: return launch_quantize<BF16>(p, a->algo, st);
-        default: return HQMQ_ERR_DTYPE;
+    return HQMQ_OK;
+}
+
+static int launch_one_tensor(const QParams &p, int dtype, int algo, hipStream_t st) {
+    switch (dtype) {
+        case HQMQ_F32: return launch_quantize<F32>(p, algo, st);
+        case HQMQ_F16: return launch_quantize<F16>(p, algo, st);
+        default: return launch_quantize<BF16>(p, algo, st);
     }
+}
+
+extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
+    QParams p;
+    bool empty;
+    const int rc = fill_qparams(a, &p, &empty);
+    if (rc || empty) return rc;
+    return launch_one_tensor(p, a->dtype, a->algo, (hipStream_t)stream);
+}
+
+int hqmq::quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, hipStream_t st) {
+    QParams pk, pv;
+    bool ek, ev;
+    int rc = fill_qparams(k, &pk, &ek);
+    if (rc) return rc;
+    rc = fill_qparams(v, &pv, &ev);
+    if (rc) return rc;
+    const bool same = !ek && !ev && k->dtype == v->dtype && k->B == v->B && k->H == v->H && k->T == v->T &&
+                      k->n_chunks == v->n_chunks && k->secondary_size == v->secondary_size && k->algo == 0 && v->algo == 0;
+    if (same) {
+        switch (k->dtype) {
+            case HQMQ_F32: return launch_quantize_pair<F32>(pk, pv, st);
+            case HQMQ_F16: return launch_quantize_pair<F16>(pk, pv, st);
+            default: return launch_quantize_pair<BF16>(pk, pv, st);
+        }
+    }
+    if (!ek) {
+        rc = launch_one_tensor(pk, k->dtype, k->algo, st);
+        if (rc) return rc;
+    }
+    return ev ? HQMQ_OK : launch_one_tensor(pv, v->dtype, v->algo, st);
 }

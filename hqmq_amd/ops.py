@@ -167,6 +167,61 @@ def outlier_compact(x: torch.Tensor, cache, t_off: int = 0, pos: Optional[torch.
             L.ptr(cache.sb_overflow), L.ptr(cache.sb_coord), L.stream_ptr(dev)), "hqmq_outlier_compact")
 
 
+def append_kv(k: torch.Tensor, v: torch.Tensor, k_cache, v_cache, k_joint, k_slack, v_joint, v_slack, radius_bits: int, *,
+              t_off: int = 0, pos: Optional[torch.Tensor] = None, median_mult: Optional[float] = None):
+    """Quantize the new rows k, v (B, H, T, d_h) into rows t_off.. of the two PackedTensors (shifted by pos[b]),
+    with Med-C extraction into their sidebands when median_mult is given.  Same results as med3x_threshold,
+    quantize and outlier_compact for K and then for V; K and V of equal shape share every launch.
+    Returns (k_count, v_count), the flagged chunks per head (int32 [H]) or (None, None)."""
+    L.require_gpu(k, "k")
+    L.require_gpu(v, "v")
+    dev = k.device
+    if pos is not None:
+        pos = pos.to(device=dev, dtype=torch.int32).contiguous()
+    keep = [pos]
+    args, counts = [], []
+    for tag, x, cache, joint, slack in (("k", k, k_cache, k_joint, k_slack), ("v", v, v_cache, v_joint, v_slack)):
+        x = _strided_x(x)
+        B, H, T, d_h = x.shape
+        if d_h % 4 != 0:
+            raise ValueError(f"d_head={d_h} not divisible by 4")
+        if joint.dtype != x.dtype or joint.shape[0] != H or not joint.is_contiguous():
+            raise ValueError("joint must be a contiguous (H, 24S, 4) table in the dtype of x")
+        a = L.AppendArgs()
+        q = a.q
+        q.x = L.ptr(x)
+        q.x_stride_b, q.x_stride_h, q.x_stride_t = x.stride(0), x.stride(1), x.stride(2)
+        q.dtype = _dt(x)
+        q.B, q.H, q.T, q.n_chunks = B, H, T, d_h // 4
+        q.joint, q.slack = L.ptr(joint), L.ptr(slack)
+        q.secondary_size, q.radius_bits, q.algo = joint.shape[1] // 24, radius_bits, 0
+        q.main_plane, q.aux_plane, q.scale_plane = L.ptr(cache.main), L.ptr(cache.aux), L.ptr(cache.scale)
+        q.t_cap, q.t_off = cache.t_cap, t_off
+        q.main_bits, q.aux_bits = cache.main_bits, cache.aux_bits
+        q.pos = L.ptr(pos)
+        keep += [x, joint, slack]
+        cnt = None
+        if median_mult is not None and T > 0:
+            nbytes = int(L.lib().hqmq_med3x_workspace_bytes(C.c_int(H), C.c_int(_dt(x))))
+            ws = _workspace(nbytes, dev, "med3x_" + tag)
+            med = torch.empty(H, dtype=torch.float32, device=dev)
+            thr = torch.empty(H, dtype=x.dtype, device=dev)
+            cnt = torch.zeros(H, dtype=torch.int32, device=dev)
+            keep += [ws, med, thr]
+            q.flag_plane = L.ptr(cache.flags)
+            a.median_mult = median_mult
+            a.med_workspace, a.med_workspace_bytes = L.ptr(ws), ws.numel()
+            a.median, a.thr, a.n_out = L.ptr(med), L.ptr(thr), L.ptr(cnt)
+            a.sideband, a.sb_cap = L.ptr(cache.sideband), cache.sb_cap
+            a.sb_tile_off, a.sb_count = L.ptr(cache.sb_tile_off), L.ptr(cache.sb_count)
+            a.overflow, a.sb_coord = L.ptr(cache.sb_overflow), L.ptr(cache.sb_coord)
+        args.append(a)
+        counts.append(cnt)
+    with torch.cuda.device(dev):
+        L.check(L.lib().hqmq_append_kv(C.byref(args[0]), C.byref(args[1]), L.stream_ptr(dev)), "hqmq_append_kv")
+    return counts[0], counts[1]
+
+
 def _i32(t: torch.Tensor) -> torch.Tensor:
     t = t if t.dtype == torch.int32 else t.to(torch.int32)
     return t if t.stride(-1) == 1 else t.contiguous()

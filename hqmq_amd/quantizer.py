@@ -194,8 +194,29 @@ class HQMQQuantizer(KVQuantizer):
         """Quantize the new tokens k, v (B, H, T_new, d_h) and write them behind the rows already in `cache`.
         pos (int32 [B]) gives each sequence's current length for ragged batches; the caller advances it."""
         self._check_supported()
-        self._append_one(cache.K, k, layer_idx, 0, pos)
-        self._append_one(cache.V, v, layer_idx, 1, pos)
+        self._append_both(cache, k, v, layer_idx, pos)
+
+    def _append_both(self, cache: PackedKV, k: torch.Tensor, v: torch.Tensor, layer_idx: int, pos, median_mult=None):
+        """K and V through one call of the library (shared launches); returns the flagged-chunk counts per head."""
+        if k.shape[2] != v.shape[2]:
+            raise ValueError("k and v must bring the same number of new tokens")
+        T = k.shape[2]
+        for pt in (cache.K, cache.V):
+            if pos is None and pt.length + T > pt.t_cap:
+                raise L.HqmqError(f"cache capacity {pt.t_cap} exceeded by append of {T} rows at {pt.length}")
+            if median_mult is not None and not pt.has_outliers:
+                raise L.HqmqError("this cache was allocated without an outlier sideband")
+        if pos is None and cache.K.length != cache.V.length:      # never the case for caches filled through append()
+            return (self._append_one(cache.K, k, layer_idx, 0, pos, median_mult),
+                    self._append_one(cache.V, v, layer_idx, 1, pos, median_mult))
+        kj, ks = self._joint_and_slack(layer_idx, 0, k)
+        vj, vs = self._joint_and_slack(layer_idx, 1, v)
+        t_off = 0 if pos is not None else cache.K.length
+        counts = ops.append_kv(k, v, cache.K, cache.V, kj, ks, vj, vs, self.radius_bits, t_off=t_off, pos=pos,
+                               median_mult=median_mult)
+        if pos is None:
+            cache.K.length = cache.V.length = t_off + T
+        return counts
 
 
 class _OutlierStats:
@@ -301,9 +322,10 @@ class OutlierAwareHQMQQuantizer(KVQuantizer, _OutlierStats):
         """Quantize-and-append with Med-C extraction; the median is over the chunks of this call, per head."""
         self._require_median_mode()
         self.inner._check_supported()
-        for pt, x, kv in ((cache.K, k, 0), (cache.V, v, 1)):
-            count = self.inner._append_one(pt, x, layer_idx, kv, pos, median_mult=self.median_mult)
-            self._note(count, x.numel() // 4)
+        counts = self.inner._append_both(cache, k, v, layer_idx, pos, median_mult=self.median_mult)
+        for count, x in zip(counts, (k, v)):
+            if count is not None:
+                self._note(count, x.numel() // 4)
 
 
 class OutlierAwareGenericQuantizer(KVQuantizer, _OutlierStats):

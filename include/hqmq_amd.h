@@ -127,6 +127,25 @@ int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, 
                          const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off, int32_t *sb_count,
                          int32_t *overflow, uint16_t *sb_coord, void *stream);
 
+/* One append of new K and V rows to a packed cache: Med3x threshold (when median_mult > 0), quantize + pack,
+ * sideband compaction, for both tensors.  The results are those of hqmq_med3x_threshold, hqmq_quantize and
+ * hqmq_outlier_compact called in that order for K and then for V (what KVQuantizer.quantize_K / quantize_V of
+ * src/quantizers/base.py:19-27 do one after the other, src/model_utils.py:22-32); when K and V have the same shape
+ * every stage is one launch shared by the two tensors, which halves the time of a single-token append.
+ *   q            as for hqmq_quantize; with median_mult > 0, q.thr is ignored (thr below is used) and q.flag_plane
+ *                is required
+ *   median_mult  0: no outlier extraction (the fields below are not read) */
+typedef struct hqmq_append_args {
+    hqmq_quantize_args q;
+    float median_mult;
+    void *med_workspace; int64_t med_workspace_bytes;  /* hqmq_med3x_workspace_bytes(H, dtype) */
+    float *median; void *thr; int32_t *n_out;          /* [H] outputs: fp32, D, int32 (n_out may be NULL) */
+    void *sideband; int64_t sb_cap;
+    int32_t *sb_tile_off, *sb_count, *overflow;
+    uint16_t *sb_coord;                                /* may be NULL */
+} hqmq_append_args;
+int hqmq_append_kv(const hqmq_append_args *k, const hqmq_append_args *v, void *stream);
+
 /* Dense decode of unpacked codes: out = joint[h, idx] * ((rq * rs) / qmax) in D.
  * Replaces hqmq_decode_triton (src/quantizers/hqmq_kernel.py:102-132) with the
  * rounding of _decode_kv_torch (src/quantizers/hqmq_attention.py:39-65).

@@ -162,6 +162,46 @@ def test_decode_appends_keep_sideband_consistent():
     assert w._n_observations == 2 * steps
 
 
+@pytest.mark.parametrize("dn,d_h,med,ragged", [("bf16", 128, True, True), ("fp16", 64, True, False), ("fp16", 128, False, True),
+                                               ("fp32", 32, True, False)])
+def test_shared_launches_equal_single_tensor_calls(dn, d_h, med, ragged):
+    """append() sends K and V through every stage together (one launch per stage when the shapes allow it, one
+    after the other for fp32 and for bulk appends); every plane, the sideband and the counters equal those of the
+    single-tensor calls, for a bulk append followed by short ones."""
+    import hqmq
+    dt = DT[dn]
+    B, H, T0 = 3, 2, 640
+    steps = [T0, 1, 1, 5, 1, 16, 3]
+    total = sum(steps) + 8
+    inner = hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=24, radius_bits=3, device=DEV)
+    w = hqmq.with_outlier_extraction(inner) if med else inner
+    mult = w.median_mult if med else None
+    make = lambda: w.new_cache(B, total, d_h, dt, 0, sideband_frac=0.5) if med else w.new_cache(B, total, d_h, dt, 0)
+    both, single = make(), make()
+    ks = kv_input((B, H, total, d_h), dt, seed=3, outlier_p=0.05).to(DEV)
+    vs = kv_input((B, H, total, d_h), dt, seed=4, outlier_p=0.02).to(DEV)
+    pos = torch.tensor([0, 3, 7], dtype=torch.int32, device=DEV) if ragged else None
+    t = 0
+    for n_new in steps:
+        k, v = ks[:, :, t:t + n_new], vs[:, :, t:t + n_new]
+        w.append(both, k, v, 0, pos=pos)
+        inner._append_one(single.K, k, 0, 0, pos, median_mult=mult)
+        inner._append_one(single.V, v, 0, 1, pos, median_mult=mult)
+        if pos is not None:
+            pos = pos + n_new
+        t += n_new
+    names = ["main", "aux", "scale"] + (["flags", "sideband", "sb_tile_off", "sb_count", "sb_coord", "sb_overflow"] if med else [])
+    for a, b in ((both.K, single.K), (both.V, single.V)):
+        for name in names:
+            x, y = getattr(a, name), getattr(b, name)
+            if x is None and y is None:
+                continue
+            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), name
+        assert a.length == b.length
+    if med:
+        assert int(both.V.sb_count.sum()) > 0
+
+
 def test_sideband_overflow_is_reported():
     import hqmq
     w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=1, secondary_size=24, radius_bits=3, device=DEV))
