@@ -250,7 +250,8 @@ struct MedSmall {
     float *median; void *thr; int32_t *n_out;
 };
 
-template <class D>
+// NT threads (at least 256)
+template <class D, int NT>
 __device__ __forceinline__ void med_small_body(const MedSmall &a) {
     const typename D::storage *x = (const typename D::storage *)a.x;
     typename D::storage *thr = (typename D::storage *)a.thr;
@@ -266,7 +267,7 @@ __device__ __forceinline__ void med_small_body(const MedSmall &a) {
     const int per_head = B * T * n;
     if (tid == 0) { nan_count = 0; gt_count = 0; res[0] = 255; res[1] = 0; }
     __syncthreads();
-    for (int g = tid; g < per_head; g += 1024) {
+    for (int g = tid; g < per_head; g += NT) {
         const int bt = g / n, c = g - bt * n, b = bt / T, t = bt - b * T;
         const float nrm = chunk_norm<D>(x + b * xsb + h * xsh + (int64_t)t * xst + c * 4);
         if (is_nan(nrm)) { atomicAdd(&nan_count, 1u); keys[g] = 0xffffu; }
@@ -285,12 +286,12 @@ __device__ __forceinline__ void med_small_body(const MedSmall &a) {
         uint32_t hi, in_hi, lo, in_lo;
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
-        for (int g = tid; g < per_head; g += 1024) atomicAdd(&hist[keys[g] >> 8], 1u);
+        for (int g = tid; g < per_head; g += NT) atomicAdd(&hist[keys[g] >> 8], 1u);
         __syncthreads();
         find_bin256(hist, rank, wave_tot, res, hi, in_hi);
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
-        for (int g = tid; g < per_head; g += 1024)
+        for (int g = tid; g < per_head; g += NT)
             if ((uint32_t)(keys[g] >> 8) == hi) atomicAdd(&hist[keys[g] & 255u], 1u);
         __syncthreads();
         find_bin256(hist, in_hi, wave_tot, res, lo, in_lo);
@@ -309,7 +310,7 @@ __device__ __forceinline__ void med_small_body(const MedSmall &a) {
     if (n_out) {
         const float tv = thr_sh;
         uint32_t cnt = 0;
-        for (int g = tid; g < per_head; g += 1024) {
+        for (int g = tid; g < per_head; g += NT) {
             const uint32_t k = keys[g];
             const float v = (D::code == HQMQ_F16) ? __half2float(__ushort_as_half((uint16_t)k)) : __uint_as_float(k << 16);
             if (v > tv) cnt++;
@@ -320,14 +321,14 @@ __device__ __forceinline__ void med_small_body(const MedSmall &a) {
     }
 }
 
-template <class D>
-__global__ __launch_bounds__(1024) void med_small_kernel(MedSmall a) {
-    med_small_body<D>(a);
+template <class D, int NT>
+__global__ __launch_bounds__(NT) void med_small_kernel(MedSmall a) {
+    med_small_body<D, NT>(a);
 }
 // two tensors of equal shape: blockIdx.y picks one
-template <class D>
-__global__ __launch_bounds__(1024) void med_small_pair_kernel(MedSmall a, MedSmall b) {
-    med_small_body<D>(blockIdx.y ? b : a);
+template <class D, int NT>
+__global__ __launch_bounds__(NT) void med_small_pair_kernel(MedSmall a, MedSmall b) {
+    med_small_body<D, NT>(blockIdx.y ? b : a);
 }
 
 __global__ __launch_bounds__(1024) void med_select2_kernel(uint32_t *ws, int H, int64_t per_head, float mult, float *median,
@@ -366,8 +367,9 @@ __global__ void count_gt_kernel(const float *x, int64_t xsb, int64_t xsh, int64_
     if (cnt) atomicAdd(&n_out[h], cnt);
 }
 
-// One block per (b, h): walks the T new rows in order, 1024 rows per step.
-template <class D>
+// One block of NT threads per (b, h): walks the T new rows in order, NT rows per step (one wavefront for short
+// appends: its barriers cost nothing).
+template <class D, int NT>
 __device__ __forceinline__ void compact_body(const CompactCall &a) {
     using ST = typename D::storage;
     const ST *x = (const ST *)a.x;
@@ -378,7 +380,7 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
     const int32_t *pos = a.pos;
     int32_t *sb_tile_off = a.sb_tile_off, *sb_count = a.sb_count, *overflow = a.overflow;
     uint16_t *sb_coord = a.sb_coord;
-    __shared__ int scan[1024];
+    __shared__ int scan[NT];
     __shared__ int base_sh;
     const int bh = blockIdx.x, b = bh / H, h = bh - b * H;
     const int frb = (n + 7) >> 3;
@@ -386,7 +388,7 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
     const int64_t tiles = (t_cap + kTile - 1) / kTile;
     if (threadIdx.x == 0) base_sh = sb_count[bh];
     __syncthreads();
-    for (int t0 = 0; t0 < T; t0 += 1024) {
+    for (int t0 = 0; t0 < T; t0 += NT) {
         const int t = t0 + threadIdx.x;
         const int64_t row = row0 + t;
         const bool live = t < T && row < t_cap;
@@ -396,7 +398,7 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
             for (int by = 0; by < frb; by++) cnt += __popc((uint32_t)fr[by]);
         scan[threadIdx.x] = cnt;
         __syncthreads();
-        for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scan
+        for (int off = 1; off < NT; off <<= 1) {  // inclusive Hillis-Steele scan
             int v = (int)threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
             __syncthreads();
             scan[threadIdx.x] += v;
@@ -420,20 +422,20 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
             }
         }
         __syncthreads();
-        if (threadIdx.x == 1023) base_sh = base + scan[1023];
+        if (threadIdx.x == NT - 1) base_sh = base + scan[NT - 1];
         __syncthreads();
     }
     if (threadIdx.x == 0) sb_count[bh] = base_sh;
 }
 
-template <class D>
-__global__ __launch_bounds__(1024) void compact_kernel(CompactCall a) {
-    compact_body<D>(a);
+template <class D, int NT>
+__global__ __launch_bounds__(NT) void compact_kernel(CompactCall a) {
+    compact_body<D, NT>(a);
 }
 // two tensors of equal shape: blockIdx.y picks one
-template <class D>
-__global__ __launch_bounds__(1024) void compact_pair_kernel(CompactCall a, CompactCall b) {
-    compact_body<D>(blockIdx.y ? b : a);
+template <class D, int NT>
+__global__ __launch_bounds__(NT) void compact_pair_kernel(CompactCall a, CompactCall b) {
+    compact_body<D, NT>(blockIdx.y ? b : a);
 }
 
 // ---- bulk appends (whole 16-row tiles from an aligned first row): three passes with one thread per tile / row ----
@@ -527,7 +529,8 @@ static int run_med3x(const void *x, int64_t xsb, int64_t xsh, int64_t xst, int B
     const int64_t words = ws_words(H, f32);
     const int64_t per_head = (int64_t)B * T * n;
     if (!f32 && per_head <= kSmallMax) {
-        hipLaunchKernelGGL(med_small_kernel<D>, dim3(H), dim3(1024), 0, st, MedSmall{x, xsb, xsh, xst, B, T, n, mult, median, thr, n_out});
+        const MedSmall a{x, xsb, xsh, xst, B, T, n, mult, median, thr, n_out};
+        hipLaunchKernelGGL((med_small_kernel<D, 1024>), dim3(H), dim3(1024), 0, st, a);
         return hip_status(hipGetLastError());
     }
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, ws, words);
@@ -583,8 +586,10 @@ int hqmq::med3x_calls(const Med3xCall *c, int count, hipStream_t st) {
         c[0].T == c[1].T && c[0].n == c[1].n && (int64_t)c[0].B * c[0].T * c[0].n <= kSmallMax) {
         const MedSmall a{c[0].x, c[0].xsb, c[0].xsh, c[0].xst, c[0].B, c[0].T, c[0].n, c[0].mult, c[0].median, c[0].thr, c[0].n_out};
         const MedSmall b{c[1].x, c[1].xsb, c[1].xsh, c[1].xst, c[1].B, c[1].T, c[1].n, c[1].mult, c[1].median, c[1].thr, c[1].n_out};
-        if (c[0].dtype == HQMQ_F16) hipLaunchKernelGGL(med_small_pair_kernel<F16>, dim3(c[0].H, 2), dim3(1024), 0, st, a, b);
-        else hipLaunchKernelGGL(med_small_pair_kernel<BF16>, dim3(c[0].H, 2), dim3(1024), 0, st, a, b);
+        const dim3 grid(c[0].H, 2);
+        // (256 threads for a few thousand keys measured slower: 11.9 against 8.7 us, the norms load eight deep per thread)
+        if (c[0].dtype == HQMQ_F16) hipLaunchKernelGGL((med_small_pair_kernel<F16, 1024>), grid, dim3(1024), 0, st, a, b);
+        else hipLaunchKernelGGL((med_small_pair_kernel<BF16, 1024>), grid, dim3(1024), 0, st, a, b);
         return hip_status(hipGetLastError());
     }
     for (int i = 0; i < count; i++) {
@@ -633,12 +638,15 @@ static int compact_one(const CompactCall &c, hipStream_t st) {
 #undef COPY
         return hip_status(hipGetLastError());
     }
-    dim3 grid(c.B * c.H), block(1024);
-    switch (c.dtype) {
-        case HQMQ_F32: hipLaunchKernelGGL(compact_kernel<F32>, grid, block, 0, st, c); break;
-        case HQMQ_F16: hipLaunchKernelGGL(compact_kernel<F16>, grid, block, 0, st, c); break;
-        default: hipLaunchKernelGGL(compact_kernel<BF16>, grid, block, 0, st, c); break;
+    dim3 grid(c.B * c.H);
+#define LAUNCH(NT)                                                                                              \
+    switch (c.dtype) {                                                                                          \
+        case HQMQ_F32: hipLaunchKernelGGL((compact_kernel<F32, NT>), grid, dim3(NT), 0, st, c); break;          \
+        case HQMQ_F16: hipLaunchKernelGGL((compact_kernel<F16, NT>), grid, dim3(NT), 0, st, c); break;          \
+        default: hipLaunchKernelGGL((compact_kernel<BF16, NT>), grid, dim3(NT), 0, st, c); break;               \
     }
+    if (c.T <= 64) { LAUNCH(64) } else { LAUNCH(1024) }
+#undef LAUNCH
     return hip_status(hipGetLastError());
 }
 
@@ -649,12 +657,15 @@ int hqmq::compact_calls(const CompactCall *c, int count, hipStream_t st) {
     }
     if (count == 2 && c[0].T > 0 && c[0].dtype == c[1].dtype && c[0].B == c[1].B && c[0].H == c[1].H && c[0].T == c[1].T &&
         c[0].n == c[1].n && !bulk_compact(c[0]) && !bulk_compact(c[1])) {
-        dim3 grid(c[0].B * c[0].H, 2), block(1024);
-        switch (c[0].dtype) {
-            case HQMQ_F32: hipLaunchKernelGGL(compact_pair_kernel<F32>, grid, block, 0, st, c[0], c[1]); break;
-            case HQMQ_F16: hipLaunchKernelGGL(compact_pair_kernel<F16>, grid, block, 0, st, c[0], c[1]); break;
-            default: hipLaunchKernelGGL(compact_pair_kernel<BF16>, grid, block, 0, st, c[0], c[1]); break;
-        }
+        dim3 grid(c[0].B * c[0].H, 2);
+#define LAUNCH(NT)                                                                                                         \
+    switch (c[0].dtype) {                                                                                                  \
+        case HQMQ_F32: hipLaunchKernelGGL((compact_pair_kernel<F32, NT>), grid, dim3(NT), 0, st, c[0], c[1]); break;       \
+        case HQMQ_F16: hipLaunchKernelGGL((compact_pair_kernel<F16, NT>), grid, dim3(NT), 0, st, c[0], c[1]); break;       \
+        default: hipLaunchKernelGGL((compact_pair_kernel<BF16, NT>), grid, dim3(NT), 0, st, c[0], c[1]); break;            \
+    }
+        if (c[0].T <= 64) { LAUNCH(64) } else { LAUNCH(1024) }
+#undef LAUNCH
         return hip_status(hipGetLastError());
     }
     for (int i = 0; i < count; i++) {
