@@ -175,6 +175,8 @@ def append_kv(k: torch.Tensor, v: torch.Tensor, k_cache, v_cache, k_joint, k_sla
     Returns (k_count, v_count), the flagged chunks per head (int32 [H]) or (None, None)."""
     L.require_gpu(k, "k")
     L.require_gpu(v, "v")
+    if k.shape[2] == 0 and v.shape[2] == 0:        # an empty tensor has no address to pass
+        return None, None
     dev = k.device
     if pos is not None:
         pos = pos.to(device=dev, dtype=torch.int32).contiguous()

@@ -171,7 +171,7 @@ def test_shared_launches_equal_single_tensor_calls(dn, d_h, med, ragged):
     import hqmq
     dt = DT[dn]
     B, H, T0 = 3, 2, 640
-    steps = [T0, 1, 1, 5, 1, 16, 3]
+    steps = [T0, 1, 0, 1, 5, 1, 16, 3]        # an empty append changes nothing
     total = sum(steps) + 8
     inner = hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=24, radius_bits=3, device=DEV)
     w = hqmq.with_outlier_extraction(inner) if med else inner
@@ -185,8 +185,9 @@ def test_shared_launches_equal_single_tensor_calls(dn, d_h, med, ragged):
     for n_new in steps:
         k, v = ks[:, :, t:t + n_new], vs[:, :, t:t + n_new]
         w.append(both, k, v, 0, pos=pos)
-        inner._append_one(single.K, k, 0, 0, pos, median_mult=mult)
-        inner._append_one(single.V, v, 0, 1, pos, median_mult=mult)
+        if n_new:
+            inner._append_one(single.K, k, 0, 0, pos, median_mult=mult)
+            inner._append_one(single.V, v, 0, 1, pos, median_mult=mult)
         if pos is not None:
             pos = pos + n_new
         t += n_new
