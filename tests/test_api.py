@@ -170,6 +170,11 @@ def test_argument_errors_are_reported_not_launched():
     assert lib.hqmq_quantize(C.byref(a), None) == -1
     assert lib.hqmq_quantize(None, None) == -1
     assert lib.hqmq_attn_fwd(None, None) == -1
+    ak, av = L.AppendArgs(), L.AppendArgs()
+    assert lib.hqmq_append_kv(None, C.byref(av), None) == -1
+    assert lib.hqmq_append_kv(C.byref(ak), C.byref(av), None) == -1      # no input, no table
+    ak.median_mult = 3.0                                                # Med3x without a flag plane or a threshold output
+    assert lib.hqmq_append_kv(C.byref(ak), C.byref(av), None) == -1
     assert lib.hqmq_dequant(None, *([L.i64(0)] * 3), None, *([L.i64(0)] * 3), None, *([L.i64(0)] * 3), None, L.i64(0),
                             C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(1), None, None) == -1
     assert int(lib.hqmq_attn_workspace_bytes(C.c_int(1), C.c_int(32), C.c_int(1), C.c_int(128), C.c_int(64))) == 32 * 64 * 130 * 4
