@@ -137,7 +137,7 @@ def run(cfg, steps):
     res = {"config": name, "us_per_step": round(us, 2), "compressed_bytes_per_step": step_bytes,
            "GBps": round(step_bytes / us / 1e3, 1), "pct_of_hbm_roofline": round(100 * step_bytes / us / 1e3 / HBM_PEAK_GBPS, 2),
            "n_splits": n_splits, "max_abs_err_vs_dense_fp32": err, "max_abs_ref": ref_max,
-           "outlier_rate_K": round(float(cache.K.sb_count.sum()) / (B * Hkv * T * d / 4), 5),
+           "outlier_rate_K": round(float(cache.K.sb_count.sum()) / (Hkv * tokens * d / 4), 5),      # over the rows kept
            "bulk_quantize_ms_K_and_V": round(quant_ms, 2), "bulk_quantize_GTok_per_s": round(B * T / quant_ms / 1e6, 5),
            "bits_per_value": round(w.bits_per_value(), 3)}
     if cfg == 4:      # the step of config 4 also quantizes and appends one token per sequence (every context grows by 1)
