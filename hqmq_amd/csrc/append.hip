@@ -10,6 +10,7 @@ extern "C" int hqmq_append_kv(const hqmq_append_args *k, const hqmq_append_args 
     hqmq_quantize_args q[2] = {k->q, v->q};
     Med3xCall med[2];
     CompactCall cmp[2];
+    const CompactCall *with_q[2] = {nullptr, nullptr};
     int n_med = 0;
     for (int i = 0; i < 2; i++) {
         if (!(a[i]->median_mult > 0.f)) continue;
@@ -22,11 +23,20 @@ extern "C" int hqmq_append_kv(const hqmq_append_args *k, const hqmq_append_args 
         cmp[n_med] = CompactCall{q[i].x, q[i].x_stride_b, q[i].x_stride_h, q[i].x_stride_t, q[i].dtype, q[i].B, q[i].H, q[i].T,
                                  q[i].n_chunks, q[i].flag_plane, q[i].t_cap, q[i].t_off, q[i].pos, a[i]->sideband,
                                  a[i]->sb_cap, a[i]->sb_tile_off, a[i]->sb_count, a[i]->overflow, a[i]->sb_coord};
+        const int rc = check_compact(cmp[n_med]);
+        if (rc) return rc;
+        with_q[i] = &cmp[n_med];
         n_med++;
     }
     int rc = n_med ? med3x_calls(med, n_med, st) : HQMQ_OK;
     if (rc) return rc;
-    rc = quantize_two(&q[0], &q[1], st);
+    // short appends: the quantize launch compacts as well; longer ones get the compaction kernels
+    bool compacted[2];
+    rc = quantize_two(&q[0], &q[1], with_q[0], with_q[1], compacted, st);
     if (rc) return rc;
-    return n_med ? compact_calls(cmp, n_med, st) : HQMQ_OK;
+    CompactCall rest[2];
+    int n_rest = 0;
+    for (int i = 0; i < 2; i++)
+        if (with_q[i] && !compacted[i]) rest[n_rest++] = *with_q[i];
+    return n_rest ? compact_calls(rest, n_rest, st) : HQMQ_OK;
 }

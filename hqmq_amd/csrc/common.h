@@ -104,6 +104,9 @@ struct CompactCall {
 };
 int med3x_calls(const Med3xCall *c, int count, hipStream_t st);                                            // med3x.hip
 int compact_calls(const CompactCall *c, int count, hipStream_t st);                                        // med3x.hip
-int quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, hipStream_t st);                // quantize.hip
+int check_compact(const CompactCall &c);                                                                   // med3x.hip
+// ck / cv (may be NULL): the compaction that follows; compacted[i] tells whether the quantize launch did it
+int quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, const CompactCall *ck, const CompactCall *cv,
+                 bool compacted[2], hipStream_t st);                                                           // quantize.hip
 
 }  // namespace hqmq

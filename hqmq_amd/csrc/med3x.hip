@@ -607,7 +607,7 @@ extern "C" int hqmq_med3x_threshold(const void *x, int64_t x_stride_b, int64_t x
     return med3x_calls(&c, 1, (hipStream_t)stream);
 }
 
-static int check_compact(const CompactCall &c) {
+int hqmq::check_compact(const CompactCall &c) {
     if (!c.x || !c.flag_plane || !c.sideband || !c.sb_tile_off || !c.sb_count || !c.overflow) return HQMQ_ERR_NULL;
     if (c.B < 1 || c.H < 1 || c.T < 0 || c.n < 1 || c.t_cap < 1 || c.sb_cap < 1 || c.t_off < 0) return HQMQ_ERR_SHAPE;
     if (c.dtype != HQMQ_F32 && c.dtype != HQMQ_F16 && c.dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;

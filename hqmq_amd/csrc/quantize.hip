@@ -50,6 +50,12 @@ struct QParams {
     int idx_bits, main_bits, aux_bits;
     int tokens_per_block;
     int32_t *stats;
+    // sideband compaction in the same launch (compact != 0): see the end of quantize_body
+    int compact;
+    void *sideband;
+    int64_t sb_cap;
+    int32_t *sb_tile_off, *sb_count, *overflow;
+    uint16_t *sb_coord;
 };
 
 __device__ __forceinline__ void rotate_conj(const float u[4], float qw, float qx, float qy, float qz, float v[4]) {
@@ -340,9 +346,9 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
         code_sh[tid] = (uint32_t)idx | ((uint32_t)(flagged ? 0 : rq) << a.idx_bits);
         mask_sh[tid] = flagged ? 1u : 0u;
         __syncthreads();
-        if (active) {
-            const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
-            if (row < 0 || row >= a.t_cap) return;  // a bad pos[] must not write outside the plane
+        const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
+        const bool row_ok = active && row >= 0 && row < a.t_cap;  // a bad pos[] must not write outside the plane
+        if (row_ok) {
             const size_t prow = ((size_t)b * a.H + h) * a.t_cap + row;
             const uint32_t *codes = code_sh + tok_local * n;
             if (a.main_plane) {
@@ -363,6 +369,45 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(mask_sh + tok_local * n, n, 1, 0, byte);
             }
             if (a.scale_plane && c == 0) D::store((ST *)a.scale_plane + prow, rm);
+        }
+        if (a.compact) {
+            // Sideband compaction in the same launch, for appends whose new rows of a (b, h) all sit in this block
+            // (T <= tokens_per_block; n a power of two, so the lanes of a token share a wavefront).  Entries, tile
+            // offsets and counters come out as the in-order compaction kernel leaves them: flagged chunks in
+            // (row, chunk) order behind the entries already there, the offset of a tile = the count before its
+            // first row.
+            const bool f = row_ok && flagged;
+            const uint64_t m = __builtin_amdgcn_ballot_w64(f);
+            const int lane = tid & 63;
+            const uint64_t tok_bits = n == 64 ? ~0ull : ((1ull << n) - 1ull) << ((lane / n) * n);
+            const int before_c = __popcll(m & tok_bits & ((1ull << lane) - 1ull));
+            int *cnt_sh = reinterpret_cast<int *>(radius_sh);           // free since the scales were taken
+            if (c == 0 && tok_local < a.tokens_per_block) cnt_sh[tok_local] = __popcll(m & tok_bits);
+            const size_t bhs = (size_t)b * a.H + h;
+            const int base = a.sb_count[bhs];                           // read by every thread before the barrier,
+            __syncthreads();                                            // rewritten by one thread after it
+            int mine = base, total = base;
+            for (int i = 0; i < a.T; i++) {
+                const int ci = cnt_sh[i];
+                if (i < tok_local) mine += ci;
+                total += ci;
+            }
+            if (row_ok) {
+                const int64_t tiles = (a.t_cap + kTile - 1) / kTile;
+                if (c == 0 && (row & (kTile - 1)) == 0) a.sb_tile_off[bhs * tiles + (row >> 4)] = mine;
+                if (f) {
+                    const int k = mine + before_c;
+                    if (k < a.sb_cap) {
+                        const ST *xp = (const ST *)a.x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst + c * 4;
+                        ST *dst = (ST *)a.sideband + (bhs * a.sb_cap + k) * 4;
+                        for (int j = 0; j < 4; j++) dst[j] = xp[j];
+                        if (a.sb_coord) a.sb_coord[bhs * a.sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
+                    } else {
+                        *a.overflow = 1;
+                    }
+                }
+            }
+            if (tid == 0) a.sb_count[bhs] = total;
         }
     }
 }
@@ -440,7 +485,19 @@ static int fill_qparams(const hqmq_quantize_args *a, QParams *out, bool *empty) 
     p.idx_bits = ib; p.main_bits = packed ? a->main_bits : mb; p.aux_bits = packed ? a->aux_bits : ab;
     p.tokens_per_block = kQThreads / a->n_chunks;
     p.stats = a->stats;
+    p.compact = 0;
+    p.sideband = nullptr; p.sb_cap = 0; p.sb_tile_off = p.sb_count = p.overflow = nullptr; p.sb_coord = nullptr;
     return HQMQ_OK;
+}
+
+// The compaction of a short append can ride in the quantize launch: all new rows of a (b, h) in one block, the
+// lanes of a token inside one wavefront, Med3x flags being written.
+static bool take_compaction(QParams &p, const CompactCall *c) {
+    if (!c || !p.thr || !p.flag_plane || p.T > p.tokens_per_block || (p.n & (p.n - 1)) || p.n > 64) return false;
+    p.compact = 1;
+    p.sideband = c->sideband; p.sb_cap = c->sb_cap; p.sb_tile_off = c->sb_tile_off; p.sb_count = c->sb_count;
+    p.overflow = c->overflow; p.sb_coord = c->sb_coord;
+    return true;
 }
 
 static int launch_one_tensor(const QParams &p, int dtype, int algo, hipStream_t st) {
@@ -459,13 +516,16 @@ extern "C" int hqmq_quantize(const hqmq_quantize_args *a, void *stream) {
     return launch_one_tensor(p, a->dtype, a->algo, (hipStream_t)stream);
 }
 
-int hqmq::quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, hipStream_t st) {
+int hqmq::quantize_two(const hqmq_quantize_args *k, const hqmq_quantize_args *v, const CompactCall *ck, const CompactCall *cv,
+                       bool compacted[2], hipStream_t st) {
     QParams pk, pv;
     bool ek, ev;
     int rc = fill_qparams(k, &pk, &ek);
     if (rc) return rc;
     rc = fill_qparams(v, &pv, &ev);
     if (rc) return rc;
+    compacted[0] = !ek && take_compaction(pk, ck);
+    compacted[1] = !ev && take_compaction(pv, cv);
     const bool same = !ek && !ev && k->dtype == v->dtype && k->B == v->B && k->H == v->H && k->T == v->T &&
                       k->n_chunks == v->n_chunks && k->secondary_size == v->secondary_size && k->algo == 0 && v->algo == 0;
     if (same) {

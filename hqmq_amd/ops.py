@@ -129,7 +129,7 @@ def med3x_threshold(x: torch.Tensor, mult: float = 3.0, want_count: bool = True)
     ws = _workspace(nbytes, dev, "med3x")
     med = torch.empty(H, dtype=torch.float32, device=dev)
     thr = torch.empty(H, dtype=x.dtype, device=dev)
-    cnt = torch.zeros(H, dtype=torch.int32, device=dev) if want_count else None
+    cnt = torch.empty(H, dtype=torch.int32, device=dev) if want_count else None     # written for every head
     with torch.cuda.device(dev):
         L.check(L.lib().hqmq_med3x_threshold(
             L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
@@ -208,7 +208,7 @@ def append_kv(k: torch.Tensor, v: torch.Tensor, k_cache, v_cache, k_joint, k_sla
             ws = _workspace(nbytes, dev, "med3x_" + tag)
             med = torch.empty(H, dtype=torch.float32, device=dev)
             thr = torch.empty(H, dtype=x.dtype, device=dev)
-            cnt = torch.zeros(H, dtype=torch.int32, device=dev)
+            cnt = torch.empty(H, dtype=torch.int32, device=dev)      # every path of the library writes all H counts
             keep += [ws, med, thr]
             q.flag_plane = L.ptr(cache.flags)
             a.median_mult = median_mult
