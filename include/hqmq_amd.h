@@ -131,7 +131,8 @@ int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, 
  * sideband compaction, for both tensors.  The results are those of hqmq_med3x_threshold, hqmq_quantize and
  * hqmq_outlier_compact called in that order for K and then for V (what KVQuantizer.quantize_K / quantize_V of
  * src/quantizers/base.py:19-27 do one after the other, src/model_utils.py:22-32); when K and V have the same shape
- * every stage is one launch shared by the two tensors, which halves the time of a single-token append.
+ * every stage is one launch shared by the two tensors, and for appends of at most 256 / n_chunks rows (n_chunks a
+ * power of two) the quantize launch also does the compaction: a single-token append is two launches, not six.
  *   q            as for hqmq_quantize; with median_mult > 0, q.thr is ignored (thr below is used) and q.flag_plane
  *                is required
  *   median_mult  0: no outlier extraction (the fields below are not read) */
