@@ -123,20 +123,39 @@ __device__ int brute_argmax(const float u[4], const typename D::storage *jh, int
 
 // Little-endian bit stream of `w`-bit fields (field i = vals[base + i] >> shift, masked)
 // -> output byte `byte` of the row.
-__device__ __forceinline__ uint8_t gather_byte(const uint32_t *vals, int count, int w, int shift, int byte) {
+template <int W>
+__device__ __forceinline__ uint8_t gather_byte_w(const uint32_t *vals, int count, int w, int shift, int byte) {
+    const int ww = W ? W : w;       // W != 0: the width is a constant and the divisions below fold into shifts
     uint32_t out = 0;
-    uint32_t fmask = (w >= 32) ? 0xffffffffu : ((1u << w) - 1u);
+    uint32_t fmask = (ww >= 32) ? 0xffffffffu : ((1u << ww) - 1u);
+#pragma unroll
     for (int bit = 0; bit < 8; bit++) {
         int pos = byte * 8 + bit;
-        int i = pos / w, o = pos - i * w;
+        int i = pos / ww, o = pos - i * ww;
         if (i < count) out |= ((((vals[i] >> shift) & fmask) >> o) & 1u) << bit;
     }
     return (uint8_t)out;
 }
+__device__ __forceinline__ uint8_t gather_byte(const uint32_t *vals, int count, int w, int shift, int byte) {
+    switch (w) {        // the widths the layout rule produces (main 8 / 12, aux 1..3, flags 1)
+        case 1: return gather_byte_w<1>(vals, count, w, shift, byte);
+        case 2: return gather_byte_w<2>(vals, count, w, shift, byte);
+        case 3: return gather_byte_w<3>(vals, count, w, shift, byte);
+        case 8: return gather_byte_w<8>(vals, count, w, shift, byte);
+        case 12: return gather_byte_w<12>(vals, count, w, shift, byte);
+        default: return gather_byte_w<0>(vals, count, w, shift, byte);
+    }
+}
 
-template <class D, int ALGO>
+// SPLIT (single-token appends, 16-bit dtypes, n a power of two): the block's 256 / n token slots all hold the one new
+// token of (b, h) and share its secondaries between them: slot w scores s = w, w + slots, ...  A decode-step append is
+// one wavefront's serial instruction stream otherwise; this divides the search part of it by the number of slots.
+// The slots' candidates are merged exactly: the filter threshold comes from the maximum over all slots, the winner
+// is the highest exact score with the lowest index, as in the unsplit search.
+template <class D, int ALGO, bool SPLIT = false>
 __device__ __forceinline__ void quantize_body(const QParams &a) {
     using ST = typename D::storage;
+    static_assert(!SPLIT || (ALGO == 0 && D::code != HQMQ_F32), "the split search is the MFMA search");
     extern __shared__ float sec[];  // [S][4] secondaries, then [S][4] fp16 columns of their rotation matrices
     uint2 *rot = reinterpret_cast<uint2 *>(sec + 4 * a.S);
     __shared__ float radius_sh[kQThreads];
@@ -148,9 +167,11 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
     const int tid = threadIdx.x;
     const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
     const int n = a.n, S = a.S, K = 24 * S;
-    const int tok_local = tid / n, c = tid - tok_local * n;
-    const int t = blockIdx.x * a.tokens_per_block + tok_local;
+    const int tok_local = tid / n, c = tid - tok_local * n;       // SPLIT: tok_local is the slot
+    const int t = SPLIT ? (int)blockIdx.x : blockIdx.x * a.tokens_per_block + tok_local;
     const bool active = tok_local < a.tokens_per_block && t < a.T;
+    const bool writer = !SPLIT || tok_local == 0;                 // one slot stores the results
+    const int slots = SPLIT ? kQThreads / n : 1, s_first = SPLIT ? tok_local : 0;
     const ST *jh = (const ST *)a.joint + (size_t)h * K * 4;
 
     for (int i = tid; i < S * 4; i += kQThreads) sec[i] = D::load(jh + i);  // rows k = s are q_s itself
@@ -204,10 +225,10 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             // for every block, lane i holds column i), B = the lane's own direction, D = its rotated chunk.
             const half4 ub = half4{(_Float16)us[0], (_Float16)us[1], (_Float16)us[2], (_Float16)us[3]};
             const uint2 *acol = rot + (tid & 3);
-            uint2 a_next = acol[0];
-            for (int s = 0; s < S; s++) {
+            uint2 a_next = acol[4 * min(s_first, S - 1)];
+            for (int s = s_first; s < S; s += slots) {
                 const half4 am = __builtin_bit_cast(half4, a_next);
-                a_next = acol[4 * min(s + 1, S - 1)];           // the next column is on its way during this one
+                a_next = acol[4 * min(s + slots, S - 1)];       // the next column is on its way during this one
                 const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 const float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
                 asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
@@ -229,6 +250,15 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 }
             }
         }
+        if (SPLIT) {        // the maximum over all slots of this chunk (every slot holds the same direction)
+            float *m2_sh = reinterpret_cast<float *>(code_sh);
+            m2_sh[tid] = m2;
+            __syncthreads();
+            for (int w = 0; w < slots; w++) m2 = fmaxf(m2, m2_sh[w * n + c]);
+            __syncthreads();
+        }
+        float bs = -INFINITY;
+        int bk = 0x7fffffff;
         if (search) {
             if (cnt > kSCap) brute = true;
             const float thr2 = m2 - margin2;
@@ -273,8 +303,6 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 if (kcnt > kKCap) brute = true;
             }
             if (!brute) {
-                float bs = -INFINITY;
-                int bk = 0x7fffffff;
                 for (int i = 0; i < kcnt; i++) {
                     const int k = klist[i][tid];
                     const float sc = ref_score<D>(u, jh + (size_t)k * 4);
@@ -284,6 +312,30 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             }
         }
         if (brute) idx = brute_argmax<D>(u, jh, K);
+        if (SPLIT) {
+            // merge the slots: a slot that fell back to the exhaustive search holds the answer; otherwise the highest
+            // exact score wins, the lowest index among equals; no candidate anywhere (all-zero direction) -> index 0
+            float *bs_sh = reinterpret_cast<float *>(code_sh);
+            int *bk_sh = reinterpret_cast<int *>(mask_sh);
+            bs_sh[tid] = bs;
+            bk_sh[tid] = brute ? (idx | (int)0x80000000) : (search ? bk : 0x7fffffff);
+            __syncthreads();
+            float ms = -INFINITY;
+            int mk = 0x7fffffff;
+            bool exact = false;
+            for (int w = 0; w < slots; w++) {
+                const int kw = bk_sh[w * n + c];
+                const float sw = bs_sh[w * n + c];
+                if (kw < 0) {
+                    if (!exact) { exact = true; mk = kw & 0x7fffffff; }
+                } else if (!exact && kw != 0x7fffffff && (sw > ms || (sw == ms && kw < mk))) {
+                    ms = sw;
+                    mk = kw;
+                }
+            }
+            idx = mk == 0x7fffffff ? 0 : mk;
+            __syncthreads();
+        }
         if (a.stats && active) {
             if (brute) atomicAdd(a.stats, 1);
             if (search && !brute) atomicAdd(a.stats + 1, cnt);
@@ -321,7 +373,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
     bool flagged = false;
     if (a.thr) flagged = nrm > D::load((const ST *)a.thr + h);
 
-    if (active) {
+    if (active && writer) {
         const size_t o = (((size_t)b * a.H + h) * a.T + t) * n + c;
         if (a.idx_out) a.idx_out[o] = idx;
         if (a.rq_out) a.rq_out[o] = rq;
@@ -347,7 +399,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
         mask_sh[tid] = flagged ? 1u : 0u;
         __syncthreads();
         const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
-        const bool row_ok = active && row >= 0 && row < a.t_cap;  // a bad pos[] must not write outside the plane
+        const bool row_ok = active && writer && row >= 0 && row < a.t_cap;  // a bad pos[] must not write outside the plane
         if (row_ok) {
             const size_t prow = ((size_t)b * a.H + h) * a.t_cap + row;
             const uint32_t *codes = code_sh + tok_local * n;
@@ -419,15 +471,31 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
 
 // The K and the V rows of one append in one launch (same shapes): blockIdx.z picks the tensor.  A single-token
 // append is latency-bound (32 lanes per block for a few microseconds), so the two run side by side for free.
-template <class D>
+template <class D, bool SPLIT>
 __global__ __launch_bounds__(kQThreads) void quantize_pair_kernel(QParams k, QParams v) {
-    quantize_body<D, 0>(blockIdx.z ? v : k);
+    quantize_body<D, 0, SPLIT>(blockIdx.z ? v : k);
+}
+template <class D>
+__global__ __launch_bounds__(kQThreads) void quantize_split_kernel(QParams a) {
+    quantize_body<D, 0, true>(a);
+}
+
+// one new token per sequence, 16-bit dtype, the lanes of a token inside a wavefront: the split search
+template <class D>
+static bool use_split(const QParams &p, int algo) {
+    return sizeof(typename D::storage) == 2 && algo == 0 && p.T == 1 && p.n >= 4 && p.n <= 64 && !(p.n & (p.n - 1));
 }
 
 template <class D>
 static int launch_quantize(const QParams &p, int algo, hipStream_t st) {
     dim3 grid((p.T + p.tokens_per_block - 1) / p.tokens_per_block, p.B * p.H), block(kQThreads);
     size_t shmem = (size_t)p.S * 4 * sizeof(float) + (size_t)p.S * 4 * sizeof(uint2);
+    if constexpr (sizeof(typename D::storage) == 2) {
+        if (use_split<D>(p, algo)) {
+            hipLaunchKernelGGL(quantize_split_kernel<D>, grid, block, shmem, st, p);
+            return hip_status(hipGetLastError());
+        }
+    }
     if (algo == 1) hipLaunchKernelGGL((quantize_kernel<D, 1>), grid, block, shmem, st, p);
     else hipLaunchKernelGGL((quantize_kernel<D, 0>), grid, block, shmem, st, p);
     return hip_status(hipGetLastError());
@@ -437,7 +505,13 @@ template <class D>
 static int launch_quantize_pair(const QParams &k, const QParams &v, hipStream_t st) {
     dim3 grid((k.T + k.tokens_per_block - 1) / k.tokens_per_block, k.B * k.H, 2), block(kQThreads);
     size_t shmem = (size_t)k.S * 4 * sizeof(float) + (size_t)k.S * 4 * sizeof(uint2);
-    hipLaunchKernelGGL(quantize_pair_kernel<D>, grid, block, shmem, st, k, v);
+    if constexpr (sizeof(typename D::storage) == 2) {
+        if (use_split<D>(k, 0) && use_split<D>(v, 0)) {
+            hipLaunchKernelGGL((quantize_pair_kernel<D, true>), grid, block, shmem, st, k, v);
+            return hip_status(hipGetLastError());
+        }
+    }
+    hipLaunchKernelGGL((quantize_pair_kernel<D, false>), grid, block, shmem, st, k, v);
     return hip_status(hipGetLastError());
 }
 

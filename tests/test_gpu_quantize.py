@@ -87,6 +87,52 @@ def test_adversarial_ties(dn):
     assert torch.equal(got["idx"].cpu(), want["idx"]) and torch.equal(got["rq"].cpu(), want["rq"])
 
 
+@pytest.mark.parametrize("S,b_r", CODEBOOKS)
+@pytest.mark.parametrize("dn", ["fp16", "bf16"])
+@pytest.mark.parametrize("d_h", [16, 64, 128, 256])
+def test_single_token_calls_match_oracle(S, b_r, dn, d_h):
+    """Calls with one token per sequence (the decode-step append) search with the secondaries split over the
+    block's token slots; indices, radius codes and scales equal the oracle's, edge cases and ties included."""
+    ops, dt = _ops(), DT[dn]
+    H, N = 2, 160
+    raw = TO.secondary_raw(1, H, S, 9)[0, :, 0]
+    Jc = CO.joint_table(raw, dt)
+    J, slack = ops.build_joint(raw.to(DEV), dt)
+    x = kv_input((N, H, 1, d_h), dt, seed=21, outlier_p=0.02)
+    e = edge_cases(x.transpose(0, 2).contiguous())          # the helper plants along the token axis
+    x = e.transpose(0, 2).contiguous()
+    Jf = Jc[0].float()                                      # exact codewords, negatives and midpoints: ties
+    ties = torch.cat([Jf[:40], -Jf[40:80], Jf[:40] + Jf.roll(1, 0)[:40], Jf[:40] + Jf.roll(S, 0)[:40]], 0).to(dt)
+    flat = ties.reshape(-1)
+    n_tok = flat.numel() // d_h
+    x[:n_tok, 0, 0] = flat[:n_tok * d_h].reshape(n_tok, d_h)
+    want = CO.quantize(x, Jc, b_r)
+    got = ops.quantize(x.to(DEV), J, slack, b_r)
+    assert torch.equal(got["idx"].cpu(), want["idx"])
+    assert torch.equal(got["rq"].cpu(), want["rq"])
+    assert bit_equal(got["r_max"], want["r_max"])
+
+
+@pytest.mark.parametrize("S,b_r,dn,d_h", [(24, 3, "bf16", 128), (96, 4, "fp16", 128), (192, 6, "fp16", 64), (96, 4, "bf16", 32)])
+def test_token_by_token_appends_equal_one_bulk_append(S, b_r, dn, d_h):
+    """The split search of single-token appends and the bulk search leave the same planes."""
+    import hqmq
+    dt = DT[dn]
+    B, H, T = 3, 2, 37
+    q = hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=S, radius_bits=b_r, device=DEV)
+    k = edge_cases(kv_input((B, H, T, d_h), dt, seed=5, outlier_p=0.03)).to(DEV)
+    v = kv_input((B, H, T, d_h), dt, seed=6).to(DEV)
+    bulk, steps = q.new_cache(B, T, d_h, dt, 0), q.new_cache(B, T, d_h, dt, 0)
+    q.append(bulk, k, v, 0)
+    for t in range(T):
+        q.append(steps, k[:, :, t:t + 1], v[:, :, t:t + 1], 0)
+    for a, b in ((bulk.K, steps.K), (bulk.V, steps.V)):
+        for name in ("main", "aux", "scale"):
+            x, y = getattr(a, name), getattr(b, name)
+            if x is not None:
+                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), name
+
+
 def test_strided_input_and_error_paths():
     import hqmq
     ops = _ops()
