@@ -337,7 +337,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             __syncthreads();
         }
         if (a.stats && active) {
-            if (brute) atomicAdd(a.stats, 1);
+            if (brute && writer) atomicAdd(a.stats, 1);      // once per chunk, also when its slots split the search
             if (search && !brute) atomicAdd(a.stats + 1, cnt);
         }
     }
