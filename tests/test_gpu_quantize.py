@@ -107,10 +107,11 @@ def test_single_token_calls_match_oracle(S, b_r, dn, d_h):
     n_tok = flat.numel() // d_h
     x[:n_tok, 0, 0] = flat[:n_tok * d_h].reshape(n_tok, d_h)
     want = CO.quantize(x, Jc, b_r)
-    got = ops.quantize(x.to(DEV), J, slack, b_r)
+    got = ops.quantize(x.to(DEV), J, slack, b_r, want_dense=True)
     assert torch.equal(got["idx"].cpu(), want["idx"])
     assert torch.equal(got["rq"].cpu(), want["rq"])
     assert bit_equal(got["r_max"], want["r_max"])
+    assert bit_equal(got["out"], want["out"])
 
 
 @pytest.mark.parametrize("S,b_r,dn,d_h", [(24, 3, "bf16", 128), (96, 4, "fp16", 128), (192, 6, "fp16", 64), (96, 4, "bf16", 32)])
