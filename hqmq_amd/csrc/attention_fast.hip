@@ -122,6 +122,8 @@ constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chu
 constexpr int kSelOffset = kQOffset + 4096;        // outlier variants: nine rows of eight fp16, row r < 8 = unit vector r, row 8 = 0
 constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
 typedef const uint32_t __attribute__((address_space(3))) *lds_u1_ptr;
 
@@ -397,6 +399,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
     for (int e = 0; e < 4; e++) ident[e] = (_Float16)((4 * grp + e) == col ? 1.f : 0.f);
+    // bf16 caches: the verbatim sideband chunks (and the Q copy they meet) go into bf16 MFMAs as they are stored,
+    // which saves their conversion to fp16 (6 VALU per chunk); the products are exact either way
+    constexpr bool kBfEntries = FLAGS && DT == HQMQ_BF16;
+    short4v ident_bf;
+#pragma unroll
+    for (int e = 0; e < 4; e++) ident_bf[e] = (short)((4 * grp + e) == col ? 0x3F80 : 0);
 
 #pragma unroll
     for (int u = 0; u < FU; u++) {
@@ -421,7 +429,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
         for (int jj = 0; jj < CPL / 2; jj++) {
-            const uint4v q8 = __builtin_bit_cast(uint4v, qf[0][jj]);
+            uint4v q8 = __builtin_bit_cast(uint4v, qf[0][jj]);
+            if constexpr (kBfEntries) {         // the stored bf16 values
+                const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[0] * p.qsh + (int64_t)tq[0] * p.qst + grp * CPL * 4;
+                const uint2 lo = col_ok[0] ? *reinterpret_cast<const uint2 *>(qp + 8 * jj) : uint2{0, 0};
+                const uint2 hi = col_ok[0] ? *reinterpret_cast<const uint2 *>(qp + 8 * jj + 4) : uint2{0, 0};
+                q8 = uint4v{lo.x, lo.y, hi.x, hi.y};
+            }
             const int c0 = grp * CPL + 2 * jj;
             lds_tab[kQOffset / 8 + c0 * 16 + col] = uint2{q8[0], q8[1]};
             lds_tab[kQOffset / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
@@ -483,16 +497,25 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const int e0 = bs + 2 * grp;
         const uint32_t c0 = cc & (uint32_t)(n - 1), c1 = (cc >> 16) & (uint32_t)(n - 1);
         const int r0 = (cc >> 8) & 15, r1 = (cc >> 24) & 15;
-        const half4 q0 = __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(kQOffset + c0 * 128u + (uint32_t)col * 8u));
-        const half4 q1 = __builtin_bit_cast(half4, *(lds_u2_ptr)(uintptr_t)(kQOffset + c1 * 128u + (uint32_t)col * 8u));
-        const half4 h0 = chunk_to_half<DT>(x[0]), h1 = chunk_to_half<DT>(x[1]);
-        const half8 qq = cat8(q0, q1);
+        const uint2 q0r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(kQOffset + c0 * 128u + (uint32_t)col * 8u));
+        const uint2 q1r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(kQOffset + c1 * 128u + (uint32_t)col * 8u));
+        const uint2 zero_u2 = uint2{0u, 0u};
+        half4 h0 = zero_h4, h1 = zero_h4;
+        if constexpr (!kBfEntries) { h0 = chunk_to_half<DT>(x[0]); h1 = chunk_to_half<DT>(x[1]); }
+        const half8 qq = cat8(__builtin_bit_cast(half4, q0r), __builtin_bit_cast(half4, q1r));
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             if (bs < off[u + 1] && bs + 8 > off[u]) {        // wave-uniform: the batch meets tile u
                 const bool v0 = e0 >= off[u] && e0 < off[u + 1] && r0 == col;
                 const bool v1 = e0 + 1 >= off[u] && e0 + 1 < off[u + 1] && r1 == col;
-                so[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(v0 ? h0 : zero_h4, v1 ? h1 : zero_h4), qq, so[u], 0, 0, 0);
+                if constexpr (kBfEntries) {
+                    const uint2 a0 = v0 ? x[0] : zero_u2, a1 = v1 ? x[1] : zero_u2;
+                    so[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, uint4v{a0.x, a0.y, a1.x, a1.y}),
+                                                                    __builtin_bit_cast(bf16x8, uint4v{q0r.x, q0r.y, q1r.x, q1r.y}),
+                                                                    so[u], 0, 0, 0);
+                } else {
+                    so[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(v0 ? h0 : zero_h4, v1 ? h1 : zero_h4), qq, so[u], 0, 0, 0);
+                }
             }
         }
     };
@@ -533,14 +556,19 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const bool mine = ok && (int)(t >> 2) == grp;
         const uint4v sel = *(lds_u4_ptr)(uintptr_t)(kSelOffset + (mine ? slot : 8u) * 16u);
         const half4 pg = pack4(__builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0));
-        const half4 h = chunk_to_half<DT>(x);
+        half4 h = zero_h4;
+        if constexpr (!kBfEntries) h = chunk_to_half<DT>(x);
         const bool owner = ok && (int)(ch / CPL) == grp;
         const int jq = (int)(ch % CPL);
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             const bool mj = owner && jq == j;
             if (__builtin_amdgcn_ballot_w64(mj) != 0) {
-                const float4v tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
+                float4v tr;
+                if constexpr (kBfEntries)
+                    tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, mj ? x : uint2{0u, 0u}), ident_bf, zero4, 0, 0, 0);
+                else
+                    tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
                 acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
             }
         }
