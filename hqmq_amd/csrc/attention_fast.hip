@@ -424,7 +424,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     }
     if (FLAGS && threadIdx.x >= 64 && threadIdx.x < 100) {
         const uint32_t w = threadIdx.x - 64, row = w >> 2, d = w & 3;
-        reinterpret_cast<uint32_t *>(lds_tab)[kSelOffset / 4 + w] = (row < 8 && (row >> 1) == d) ? 0x3C00u << (16 * (row & 1)) : 0u;
+        // the selector rows carry qmax instead of 1: the gathered probabilities come out scaled for the verbatim
+        // chunks (whose 1 / qmax is applied with everything else in the epilogue) at no cost
+        const uint32_t one = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(float)p.qmax);
+        reinterpret_cast<uint32_t *>(lds_tab)[kSelOffset / 4 + w] = (row < 8 && (row >> 1) == d) ? one << (16 * (row & 1)) : 0u;
     }
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
@@ -532,8 +535,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     };
     // V side, also from the entry list, sixteen entries of the half-step per batch (lane 16 * grp + col holds
     // entry `col`):
-    //   Pg[e][column] = P[token(e)][column]      one 16x16x32 MFMA: A = the unit vector of the entry's token slot
-    //                                            (LDS rows), B = the unscaled probabilities of the 32 tokens;
+    //   Pg[e][column] = qmax P[token(e)][column] one 16x16x32 MFMA: A = qmax times the unit vector of the entry's token
+    //                                            slot (LDS rows), B = the unscaled probabilities of the 32 tokens;
     //   for every chunk position j in use:       X_j^T by the transposing MFMA (A = the entry's chunk in the row
     //   acc[j] += X_j^T . Pg                     group that owns it, else zero), then one 16x16x16 MFMA over entries.
     constexpr int kVPre = CPL >= 8 ? 2 : 1;
@@ -644,10 +647,11 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                     pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[cgi][u][e], c, mc));
                     l_run[cgi] += pe[e];
                 }
-                const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(h.vs[u].x);
-                const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(h.vs[u].y);
+                const half2v u01 = half2v{(_Float16)pe[0], (_Float16)pe[1]}, u23 = half2v{(_Float16)pe[2], (_Float16)pe[3]};
+                const half2v p01 = u01 * scale_h2<DT>(h.vs[u].x);
+                const half2v p23 = u23 * scale_h2<DT>(h.vs[u].y);
                 pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
-                if (FLAGS) pTo[u] = half4{(_Float16)(pe[0] * qmaxf), (_Float16)(pe[1] * qmaxf), (_Float16)(pe[2] * qmaxf), (_Float16)(pe[3] * qmaxf)};
+                if (FLAGS) pTo[u] = half4{u01[0], u01[1], u23[0], u23[1]};      // unscaled: the selector rows hold qmax
             }
             pp[cgi] = cat8(pT[0], pT[1]);
         }
