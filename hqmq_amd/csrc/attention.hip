@@ -306,6 +306,9 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
 // One block per output row, one thread per element.  Every thread loads the (m, l, acc[e]) of up to 32 splits in
 // one batch of independent loads (the m and l of a split are the same addresses in all threads: broadcasts) and
 // merges them in registers, so the kernel costs one round trip to memory per 32 splits; no LDS, no barrier.
+// SC: splits loaded per batch of independent loads (the smallest of 4, 8, 32 that covers n_splits, so that few
+// splits do not pay for 32 predicated loads)
+template <int SC>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
                                                            int n_splits, int64_t osb, int64_t osh, int64_t ost) {
     const int64_t row = blockIdx.x;
@@ -313,7 +316,6 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void
     if (e >= d_h) return;
     const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
     const float *base = ws + (size_t)row * n_splits * (d_h + 2);
-    constexpr int SC = 32;
     float M = -INFINITY, L = 0.f, A = 0.f;
     for (int s0 = 0; s0 < n_splits; s0 += SC) {
         float ms[SC], ls[SC], as[SC];
@@ -406,7 +408,8 @@ extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int 
     if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3((d_h + 63) / 64 * 64), 0, (hipStream_t)stream,
+    auto kern = n_splits <= 4 ? attn_combine_kernel<4> : n_splits <= 8 ? attn_combine_kernel<8> : attn_combine_kernel<32>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3((d_h + 63) / 64 * 64), 0, (hipStream_t)stream,
                        (const float *)workspace, O,
                        dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
