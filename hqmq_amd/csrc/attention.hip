@@ -19,6 +19,7 @@
 //     vector load per 16-token tile, a wavefront covering whole 128-byte lines of the plane;
 //   * split-KV partials (m, l, acc) go to a workspace and are merged by a second kernel.
 #include "attention_common.h"
+#include <mutex>
 
 namespace hqmq {
 
@@ -415,7 +416,7 @@ extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int 
     return hip_status(hipGetLastError());
 }
 
-extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
+static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     if (!a || !a->Q || !a->O) return HQMQ_ERR_NULL;
     const hqmq_packed *pk[2] = {&a->K, &a->V};
     for (const hqmq_packed *k : pk) {
@@ -504,4 +505,61 @@ extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) {
         rc = hqmq_attn_combine(a->workspace, a->O, a->dtype, a->B, a->H_q, a->T_q, 4 * n, n_splits, a->o_sb, a->o_sh, a->o_st,
                                stream);
     return rc;
+}
+
+extern "C" int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream) { return attn_fwd_impl(a, stream); }
+
+// ---- the entry point that allocates nothing: split partials in a static device array ----
+// Every GPU the library runs on holds its own copy of this array at its own address until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; kernels and host calls use the
+// per-device address looked up below.
+static __device__ __align__(256) unsigned char scratch[HQMQ_ATTN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// The device address of `scratch` on the current device; looked up once per device.
+int static_scratch(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HQMQ_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return HQMQ_ERR_NULL;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return HQMQ_OK;
+}
+}  // namespace
+
+extern "C" int64_t hqmq_attn_static_scratch_bytes(void) { return HQMQ_ATTN_STATIC_SCRATCH_BYTES; }
+
+extern "C" int hqmq_attn_fwd_static(const hqmq_attn_args *a, void *stream) {
+    if (!a) return HQMQ_ERR_NULL;
+    if (a->skip_combine) return HQMQ_ERR_SCRATCH;       // the partials would stay in memory the caller cannot name
+    if (a->B < 1 || a->H_q < 1 || a->H_kv < 1 || a->T_q < 1 || a->T_kv < 0 || a->n_chunks < 1) return HQMQ_ERR_SHAPE;
+    hqmq_attn_args b = *a;
+    b.n_splits = a->n_splits > 0 ? a->n_splits : hqmq_attn_pick_splits(a->B, a->H_q, a->H_kv, a->T_q, a->T_kv, a->kv_len != nullptr);
+    if (b.n_splits > 8192) return HQMQ_ERR_SHAPE;
+    b.workspace = nullptr;
+    b.workspace_bytes = 0;
+    if (b.n_splits > 1) {
+        // the partials of this call, (m, l, acc) per (row, split), are all written before they are read:
+        // nothing in the array has to start at zero
+        const int64_t need = hqmq_attn_workspace_bytes(a->B, a->H_q, a->T_q, 4 * a->n_chunks, b.n_splits);
+        if (need > (int64_t)HQMQ_ATTN_STATIC_SCRATCH_BYTES) return HQMQ_ERR_SCRATCH;
+        void *ptr = nullptr;
+        const int rc = static_scratch(&ptr);
+        if (rc) return rc;
+        b.workspace = ptr;
+        b.workspace_bytes = HQMQ_ATTN_STATIC_SCRATCH_BYTES;
+    }
+    return attn_fwd_impl(&b, stream);
 }

@@ -12,6 +12,7 @@ extern "C" const char *hqmq_status_string(int status) {
         case HQMQ_ERR_LAYOUT: return "bit widths inconsistent with the layout rules";
         case HQMQ_ERR_WORKSPACE: return "workspace too small";
         case HQMQ_ERR_ALIGN: return "a pointer or stride is not aligned as required";
+        case HQMQ_ERR_SCRATCH: return "the call does not fit the library's static scratch (8 MiB of split partials; skip_combine is not available)";
         default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
     }
 }

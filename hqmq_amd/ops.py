@@ -290,10 +290,13 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
              kv_starts: Optional[torch.Tensor] = None, batch_order: Optional[torch.Tensor] = None, causal: bool = False,
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
-             force_generic: bool = False, kernel_events: Optional[tuple] = None) -> torch.Tensor:
+             force_generic: bool = False, kernel_events: Optional[tuple] = None,
+             static_scratch: bool = False) -> torch.Tensor:
     """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each).
     kernel_events: two raw hipEvent_t handles (ints) that receive the GPU timestamps of the begin and the end of
-    the main attention kernel (profiling)."""
+    the main attention kernel (profiling).
+    static_scratch: call hqmq_attn_fwd_static, which keeps the split partials in the library's own device array
+    instead of a torch workspace (pass `out` as well and the call allocates nothing on the device)."""
     L.require_gpu(Q, "Q")
     if Q.stride(-1) != 1:
         Q = Q.contiguous()
@@ -342,6 +345,10 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     if kernel_events is not None:
         a.start_event, a.stop_event = C.c_void_p(kernel_events[0]), C.c_void_p(kernel_events[1])
     ws = None
+    if static_scratch:
+        with torch.cuda.device(dev):
+            L.check(L.lib().hqmq_attn_fwd_static(C.byref(a), L.stream_ptr(dev)), "hqmq_attn_fwd_static")
+        return O
     if n_splits > 1:
         nbytes = int(L.lib().hqmq_attn_workspace_bytes(C.c_int(B), C.c_int(Hq), C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits)))
         ws = _workspace(nbytes, dev, "attn")

@@ -48,7 +48,9 @@ enum {
     HQMQ_ERR_DTYPE = -3,     /* unknown or unsupported dtype */
     HQMQ_ERR_LAYOUT = -4,    /* bit widths inconsistent with the layout rules */
     HQMQ_ERR_WORKSPACE = -5, /* workspace too small */
-    HQMQ_ERR_ALIGN = -6      /* a pointer or stride is not aligned as required */
+    HQMQ_ERR_ALIGN = -6,     /* a pointer or stride is not aligned as required */
+    HQMQ_ERR_SCRATCH = -7    /* hqmq_attn_fwd_static: the call needs more than the library's static scratch
+                                (HQMQ_ATTN_STATIC_SCRATCH_BYTES), or asks for skip_combine */
 };
 
 int hqmq_version(void);                    /* 0xMMmmpp */
@@ -222,6 +224,21 @@ int hqmq_attn_fwd(const hqmq_attn_args *a, void *stream);
 /* Merge of the split-KV partials (m, l, acc) left in the workspace; hqmq_attn_fwd runs it unless skip_combine. */
 int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q, int T_q, int d_h, int n_splits,
                       int64_t o_sb, int64_t o_sh, int64_t o_st, void *stream);
+
+/* hqmq_attn_fwd for callers that cannot allocate or hand over scratch memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and results as hqmq_attn_fwd, except that a->workspace / a->workspace_bytes are ignored:
+ * the split-KV partials live in a device array of HQMQ_ATTN_STATIC_SCRATCH_BYTES that is part of the library's
+ * code object (every GPU the library runs on holds its own copy until the process ends).  The call allocates and
+ * frees nothing.  It returns HQMQ_ERR_SCRATCH when hqmq_attn_workspace_bytes(B, H_q, T_q, d_h, n_splits) for the
+ * chosen n_splits exceeds that size (every decode shape of the benchmark configurations fits; long chunked
+ * prefills do not: pass a smaller n_splits or use hqmq_attn_fwd) and when skip_combine is set.
+ * All calls on one GPU share the array: calls that overlap on one GPU (different streams or threads) race.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress) and must not be made under
+ * stream capture; later calls may be. */
+#define HQMQ_ATTN_STATIC_SCRATCH_BYTES (8 << 20)
+int64_t hqmq_attn_static_scratch_bytes(void);
+int hqmq_attn_fwd_static(const hqmq_attn_args *a, void *stream);
 
 #ifdef __cplusplus
 }
