@@ -43,17 +43,24 @@ def event_us(fn, iters):
 
 
 def synth(shape, dt, seed, lognormal=False, outlier_p=0.0, gain=(50.0, 200.0)):
-    g = torch.Generator(device=DEV).manual_seed(seed)
+    """Synthetic K or V (B, H, T, d): N(0, 1), optional per-channel lognormal(0, 0.5) scale, optional outlier chunks
+    (a Bernoulli(outlier_p) choice of whole chunks scaled by U(gain)).  Seeded with a CPU generator, drawn one
+    sequence at a time on the host and then moved, so that a CPU restatement can see the same inputs."""
+    g = torch.Generator().manual_seed(seed)
     B, H, T, d = shape
-    x = torch.randn(B, H, T, d, generator=g, device=DEV)
-    if lognormal:
-        x *= torch.exp(0.5 * torch.randn(B, H, 1, d, generator=g, device=DEV))
-    if outlier_p > 0:
-        n = d // 4
-        hit = torch.rand(B, H, T, n, 1, generator=g, device=DEV) < outlier_p
-        f = gain[0] + (gain[1] - gain[0]) * torch.rand(B, H, T, n, 1, generator=g, device=DEV)
-        x = torch.where(hit, x.view(B, H, T, n, 4) * f, x.view(B, H, T, n, 4)).reshape(B, H, T, d)
-    return x.to(dt)
+    out = torch.empty(B, H, T, d, dtype=dt, device=DEV)
+    chan = torch.exp(0.5 * torch.randn(H, 1, d, generator=g)) if lognormal else None
+    n = d // 4
+    for b in range(B):
+        x = torch.randn(H, T, d, generator=g)
+        if chan is not None:
+            x *= chan
+        if outlier_p > 0:
+            hit = torch.rand(H, T, n, 1, generator=g) < outlier_p
+            f = gain[0] + (gain[1] - gain[0]) * torch.rand(H, T, n, 1, generator=g)
+            x = torch.where(hit, x.view(H, T, n, 4) * f, x.view(H, T, n, 4)).reshape(H, T, d)
+        out[b] = x.to(dt).to(DEV, non_blocking=True)
+    return out
 
 
 def dense_check(Q, cache, lens, T):
@@ -111,7 +118,7 @@ def run(cfg, steps):
     lens_dev = lens.to(DEV) if lens is not None else None
     if lens is not None:
         cache.crop_(lens_dev)                    # every sequence keeps its own context; the rows behind it are free
-    Q = torch.randn(B, Hq, 1, d, generator=torch.Generator(device=DEV).manual_seed(7), device=DEV).to(dt)
+    Q = torch.randn(B, Hq, 1, d, generator=torch.Generator().manual_seed(7)).to(dt).to(DEV)
     out = torch.empty_like(Q)
     err, ref_max = dense_check(Q, cache, lens, T)
     # algorithmic bytes of one step: the valid rows of every plane + 8 B per flagged chunk in them

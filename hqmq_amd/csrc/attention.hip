@@ -471,6 +471,10 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     p.n_splits = n_splits;
     p.n_cg = (a->T_q * p.G + 15) / 16;
     p.ws = (float *)a->workspace;
+    // Workgroups go to the eight XCDs round-robin in dispatch order.  Numbering them (sequence, KV head)-fastest puts
+    // all blocks of one KV head on one XCD, whose L2 then fetches that head's two codeword tables once for all of them.
+    // Ragged batches keep the sequence-major order that batch_order relies on.
+    p.xcd_remap = (!a->kv_len && !a->batch_order && ((a->B * a->H_kv) % 8) == 0) ? 1 : 0;
     // 4 consecutive scales with one vector load: unit stride, aligned rows, and capacity rows readable
     const int salign = a->dtype == HQMQ_F32 ? 16 : 8;
     p.scale_vec = 1;

@@ -45,6 +45,7 @@ struct AttnParams {
     int n_splits, n_cg;
     int scale_vec;  // scales of 4 consecutive tokens may be read with one aligned vector load
     float *ws;      // split partials [row][split][d_h + 2]
+    int xcd_remap;  // blocks of one (sequence, KV head) share an XCD (see attn_fast_kernel)
 };
 
 __device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {

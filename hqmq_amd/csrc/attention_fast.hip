@@ -20,6 +20,7 @@ namespace hqmq {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef const uint2 __attribute__((address_space(3))) *lds_u2_ptr;
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 template <int DT>
 __device__ __forceinline__ half4 chunk_to_half(uint2 w) {
@@ -30,25 +31,47 @@ __device__ __forceinline__ half4 chunk_to_half(uint2 w) {
     return r;
 }
 
-// Both per-head tables -> LDS as fp16; every load of the block is in flight before the first store.
+// Two codewords (16 bytes) of a table in the cache dtype -> the same two as fp16
+template <int DT>
+__device__ __forceinline__ uint4v pair_to_half(uint4v w) {
+    if (DT == HQMQ_F16) return w;
+    const uint2 a = __builtin_bit_cast(uint2, chunk_to_half<DT>(uint2{w[0], w[1]}));
+    const uint2 b = __builtin_bit_cast(uint2, chunk_to_half<DT>(uint2{w[2], w[3]}));
+    return uint4v{a.x, a.y, b.x, b.y};
+}
+
+// The rest of both per-head tables (pairs k0.. of K2 / V2 pairs) -> LDS as fp16, in batches of independent loads.
 template <int DT, int NT>
-__device__ __forceinline__ void fill_tables16(uint2 *kdst, const uint2 *ksrc, int Kk, uint2 *vdst, const uint2 *vsrc, int Kv) {
-    constexpr int U = 5;
-    for (int k0 = threadIdx.x; k0 < max(Kk, Kv); k0 += NT * U) {
-        uint2 tk[U], tv[U];
+__device__ __forceinline__ void fill_tables16(uint4v *kdst, const uint4v *ksrc, int Kk2, uint4v *vdst, const uint4v *vsrc, int Kv2, int k_first) {
+    constexpr int U = 3;
+    for (int k0 = k_first + threadIdx.x; k0 < max(Kk2, Kv2); k0 += NT * U) {
+        uint4v tk[U], tv[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = k0 + u * NT;
-            tk[u] = k < Kk ? ksrc[k] : uint2{0, 0};
-            tv[u] = k < Kv ? vsrc[k] : uint2{0, 0};
+            tk[u] = ksrc[min(k, Kk2 - 1)];
+            tv[u] = vsrc[min(k, Kv2 - 1)];
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = k0 + u * NT;
-            if (k < Kk) kdst[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tk[u]));
-            if (k < Kv) vdst[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tv[u]));
+            if (k < Kk2) kdst[k] = pair_to_half<DT>(tk[u]);
+            if (k < Kv2) vdst[k] = pair_to_half<DT>(tv[u]);
         }
     }
+}
+
+// The parameter block spans several 64-byte lines of the kernel-argument segment, and the prologue reads them one
+// after the other as its address arithmetic proceeds: every first touch of a line is a miss of the scalar cache
+// that the next scalar load waits behind.  One dword of every line, requested together at the very start, turns
+// the chain of misses into one.
+__device__ __forceinline__ void touch_kernargs() {
+    typedef const uint32_t __attribute__((address_space(4))) *karg_ptr;
+    karg_ptr ka = (karg_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    uint32_t t = 0;
+#pragma unroll
+    for (int i = 0; i < (int)((sizeof(AttnParams) + 63) / 64); i++) t |= ka[16 * i];
+    asm volatile("" ::"s"(t));
 }
 
 constexpr int kFastWaves = 8;     // wavefronts per block; 12 (three per SIMD) for plain 16+0 caches with long ranges per block
@@ -119,9 +142,10 @@ __device__ __forceinline__ float scaled(float acc, uint32_t pair, int hi, float 
 // the V table at kVTabOffset, and a gather addresses them with idx * 8 (+ the instruction's immediate offset).
 constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords in front of it
 constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chunk][column] fp16 chunks, after the V table
+constexpr int kFlagsTabMax = (kQOffset - kVTabOffset) / 8;      // codewords the V slot of the outlier variants holds
+static_assert(kFlagsTabMax * 8 + kVTabOffset == kQOffset && kFlagsTabMax == 4608, "V table slot of the outlier variants");
 constexpr int kSelOffset = kQOffset + 4096;        // outlier variants: nine rows of eight fp16, row r < 8 = unit vector r, row 8 = 0
 constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
-typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
@@ -253,13 +277,24 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
+    touch_kernargs();
 
     // blocks are dispatched in grid order: batch_order lists the sequences in the order they should start
     // (longest first for ragged batches, so that no long sequence is left for the end)
-    const int slot = blockIdx.z / p.Hkv, hkv = blockIdx.z - slot * p.Hkv;
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    if (p.xcd_remap) {
+        // the hardware hands workgroups to the XCDs round-robin in linear order (x fastest): renumber so that the
+        // (sequence, KV head) index runs fastest and, with a multiple of eight of them, stays on one XCD
+        const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned r = lin / gridDim.z;
+        bz = (int)(lin - r * gridDim.z);
+        by = (int)(r / gridDim.x);
+        bx = (int)(r - (unsigned)by * gridDim.x);
+    }
+    const int slot = bz / p.Hkv, hkv = bz - slot * p.Hkv;
     const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
     const int bh = b * p.Hkv + hkv;
-    const int cg0 = blockIdx.y * NCG, sp = blockIdx.x;
+    const int cg0 = by * NCG, sp = bx;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int G = p.G;
     constexpr int n = 4 * CPL, d_h = 16 * CPL;
@@ -282,12 +317,16 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         blk_lim = max(blk_lim, col_lim[cgi]);
         if (col_ok[cgi]) lim_min = min(lim_min, col_lim[cgi]);
     }
-    for (int o = 1; o < 16; o <<= 1) {
-        blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
-        lim_min = min(lim_min, __shfl_xor(lim_min, o));
+    if (p.causal) {
+        for (int o = 1; o < 16; o <<= 1) {
+            blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
+            lim_min = min(lim_min, __shfl_xor(lim_min, o));
+        }
+        blk_lim = __builtin_amdgcn_readfirstlane(blk_lim);      // the same in every lane: all rows hold all 16 columns
+        lim_min = __builtin_amdgcn_readfirstlane(lim_min);
+    } else {
+        blk_lim = lim_min = kv_end;         // every column in range sees the whole sequence (a launched block has one)
     }
-    blk_lim = __builtin_amdgcn_readfirstlane(blk_lim);      // the same in every lane: all rows hold all 16 columns
-    lim_min = __builtin_amdgcn_readfirstlane(lim_min);
     // tokens before kv_start[b] are invisible (left padding): the walk starts at the super-tile that holds it
     const int col_start = p.kv_start ? min(max(p.kv_start[b], 0), blk_lim) : 0;
     const int blk_lo = col_start / kSuper * kSuper;
@@ -351,10 +390,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[cgi] * p.qsh + (int64_t)tq[cgi] * p.qst + grp * CPL * 4;
 #pragma unroll
         for (int j = 0; j < CPL / 2; j++) {
-            const half4 z = half4{0, 0, 0, 0};
-            const half4 lo = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
-            const half4 hi = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
-            qf[cgi][j] = cat8(lo, hi);
+            // columns out of range point at a valid row (tq = 0, first head of the group): load, then clear
+            // (an and with a lane mask, not a conditional: no branch and no wait between the loads)
+            const uint32_t keep = col_ok[cgi] ? 0xffffffffu : 0u;
+            uint2 lo = *reinterpret_cast<const uint2 *>(qp + 8 * j), hi = *reinterpret_cast<const uint2 *>(qp + 8 * j + 4);
+            lo.x &= keep; lo.y &= keep; hi.x &= keep; hi.y &= keep;
+            qf[cgi][j] = cat8(chunk_to_half<DT>(lo), chunk_to_half<DT>(hi));
         }
     }
     auto load_flags = [&](int th, FlagTile &f) {
@@ -377,23 +418,28 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // First batch of codeword-table loads (the longest dependency chain of the prologue: load, convert, LDS
     // store, barrier), then the wavefront's first super-tile; the LDS stores follow.  The Q rows were requested
     // before both so that waiting for them does not wait for the tiles.
-    constexpr int FU = 5;
-    const uint2 *ksrc = (const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4), *vsrc = (const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4);
-    const int Kk = p.Kc.K, Kv = p.Vc.K;
-    uint2 tk[FU], tv[FU];
+    // 16-byte loads of two codewords, all unconditional (clamped): straight-line code, exact wait counts
+    constexpr int FU = 3;
+    const uint4v *ksrc = (const uint4v *)((const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4));
+    const uint4v *vsrc = (const uint4v *)((const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4));
+    const int Kk2 = p.Kc.K >> 1, Kv2 = p.Vc.K >> 1;        // tables of an even number of codewords (checked at launch)
+    uint4v tk[FU], tv[FU];
 #pragma unroll
     for (int u = 0; u < FU; u++) {
         const int k = threadIdx.x + u * NT;
-        tk[u] = k < Kk ? ksrc[k] : uint2{0, 0};
-        tv[u] = k < Kv ? vsrc[k] : uint2{0, 0};
+        tk[u] = ksrc[min(k, Kk2 - 1)];
+        tv[u] = vsrc[min(k, Kv2 - 1)];
     }
 
     FastTile<NW, AB, FLAGS, NH> cur;
     FlagTile f0 = {}, f1 = {};
-    if (t_begin < t_end) {
-        if (FLAGS) load_flags(t_begin, f0);
-        load_super(t_begin, cur);
-        if (FLAGS && t_begin + STEP < t_end) load_flags(t_begin + STEP, f1);
+    {
+        // unconditional (a wavefront without a range reads a valid tile it never uses): no branch, so the waits for the
+        // table loads below count these loads as issued
+        const int t_first = min(t_begin, (int)p.t_cap - 32);
+        if (FLAGS) load_flags(t_first, f0);
+        load_super(t_first, cur);
+        if (FLAGS) load_flags(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);
     }
 
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
@@ -406,14 +452,16 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
     for (int e = 0; e < 4; e++) ident_bf[e] = (short)((4 * grp + e) == col ? 0x3F80 : 0);
 
+    {
+        uint4v *ktab4 = reinterpret_cast<uint4v *>(ktab), *vtab4 = reinterpret_cast<uint4v *>(vtab);
 #pragma unroll
-    for (int u = 0; u < FU; u++) {
-        const int k = threadIdx.x + u * NT;
-        if (k < Kk) ktab[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tk[u]));
-        if (k < Kv) vtab[k] = __builtin_bit_cast(uint2, chunk_to_half<DT>(tv[u]));
+        for (int u = 0; u < FU; u++) {
+            const int k = threadIdx.x + u * NT;
+            if (k < Kk2) ktab4[k] = pair_to_half<DT>(tk[u]);
+            if (k < Kv2) vtab4[k] = pair_to_half<DT>(tv[u]);
+        }
+        if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT>(ktab4, ksrc, Kk2, vtab4, vsrc, Kv2, FU * NT);
     }
-    if (max(Kk, Kv) > FU * NT)
-        fill_tables16<DT, NT>(ktab + FU * NT, ksrc + FU * NT, Kk - FU * NT, vtab + FU * NT, vsrc + FU * NT, Kv - FU * NT);
     // Plain variants keep two half-steps in flight.  The second one is requested only now, when the table loads
     // have come back: requested at the start it would queue in front of them and delay the whole block.
     auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
@@ -794,6 +842,11 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st
 template <int CPL, int DT>
 static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
+    // the outlier variants keep Q and the selector rows behind a smaller V slot
+    if (flags && (p.Kc.K > kFlagsTabMax || p.Vc.K > kFlagsTabMax)) return HQMQ_OK;
+    // tables are read two codewords (16 bytes) at a time
+    if ((p.Kc.K & 1) || (p.Vc.K & 1) || (p.Kc.jsh & 7) || (p.Vc.jsh & 7) || (((uintptr_t)p.Kc.joint | (uintptr_t)p.Vc.joint) & 15))
+        return HQMQ_OK;
     *handled = true;
     // long ranges per block (large batches): twelve wavefronts per block, three per SIMD, stream 3-12 % faster; the
     // variants that need more than 168 registers and short launches stay at eight

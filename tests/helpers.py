@@ -106,3 +106,58 @@ def assert_attention_close(got, ref_d, ref_x, a_abs, base=2e-3, what=""):
                                  f"|O - ref| max {float(e_d.max()):.3e} (over by {w2:.3e}), "
                                  f"reference rounding spread max {float(spread.max()):.3e}")
     return float(e_d.max())
+
+
+def unpack_planes(pt, b: int, L: int):
+    """Independent reader (plain torch ops, on the cache's device) of rows [0, L) of sequence b of a PackedTensor:
+    (idx, rq) int64 of shape (H, L, n) and the flag bits as a bool tensor of the same shape (None without Med3x).
+    Little-endian bit streams: main_bits per code in the main row, the remaining aux_bits in the aux row."""
+    n, ib, mb, ab = pt.n, pt.idx_bits, pt.main_bits, pt.aux_bits
+    dev = pt.main.device
+
+    def fields(plane, width):
+        H = plane.shape[0]
+        bit = (plane.unsqueeze(-1).to(torch.int32) >> torch.arange(8, device=dev, dtype=torch.int32)) & 1
+        bit = bit.reshape(H, L, -1)[..., :n * width].reshape(H, L, n, width).to(torch.int64)
+        return (bit << torch.arange(width, device=dev)).sum(-1)
+
+    code = fields(pt.main[b, :, :L], mb)
+    if ab:
+        code = code | (fields(pt.aux[b, :, :L], ab) << mb)
+    flags = fields(pt.flags[b, :, :L], 1).bool() if pt.flags is not None else None
+    return code & ((1 << ib) - 1), code >> ib, flags
+
+
+def exact_dense(pt, b: int, L: int, x=None) -> torch.Tensor:
+    """fp32 (H, L, d_h) decode of sequence b without any rounding to the cache dtype: joint[idx] * (rq * rs / qmax),
+    flagged chunks verbatim from x (H, L, d_h), the tensor that was quantized."""
+    idx, rq, flags = unpack_planes(pt, b, L)
+    H, n = pt.H, pt.n
+    J = pt.joint.float()
+    cw = torch.stack([J[h][idx[h]] for h in range(H)])                              # (H, L, n, 4)
+    rad = rq.float() * pt.scale[b, :, :L].float().unsqueeze(-1) / float(pt.qmax)
+    d = cw * rad.unsqueeze(-1)
+    if flags is not None:
+        assert x is not None
+        d = torch.where(flags.unsqueeze(-1), x.float().view(H, L, n, 4), d)
+    return d.reshape(H, L, 4 * n)
+
+
+def gpu_attention_refs(Qb, K_D, V_D, K_x, V_x):
+    """One sequence, decode: Qb (H_q, d), dense caches (H_kv, L, d).  Returns (ref over the D-rounded cache, ref over
+    the unrounded cache, attention-weighted |V|), fp32 on the GPU (softmax in float64)."""
+    Hq, d = Qb.shape
+    Hkv = K_D.shape[0]
+    g = Hq // Hkv
+    q = Qb.double().view(Hkv, g, d)
+
+    def attend(K, V, Vabs=None):
+        p = torch.softmax(torch.einsum("hgd,hkd->hgk", q, K.double()) * d ** -0.5, dim=-1)
+        o = torch.einsum("hgk,hkd->hgd", p, V.double()).reshape(Hq, d).float()
+        if Vabs is None:
+            return o
+        return o, torch.einsum("hgk,hkd->hgd", p, Vabs.double()).reshape(Hq, d).float()
+
+    ref_d = attend(K_D, V_D)
+    ref_x, a_abs = attend(K_x, V_x, V_x.abs())
+    return ref_d, ref_x, a_abs

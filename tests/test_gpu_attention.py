@@ -13,7 +13,7 @@ import torch
 from oracle import c_oracle as CO
 from oracle import torch_oracle as TO
 from tests.helpers import (DT, assert_attention_close, attention_refs, attn_tolerance, bit_equal, dense_from_codes,
-                           kv_input, unbits)
+                           exact_dense, gpu_attention_refs, kv_input, unbits, unpack_planes)
 from tests.test_oracle import ATTN_CASES, load_attn_case
 
 pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
@@ -142,7 +142,7 @@ def test_torch_sdpa_agrees_on_the_same_cache():
     assert (O.float() - ref.float()).abs().max().item() < 2e-3
 
 
-@pytest.mark.parametrize("T", [4096, 32768])
+@pytest.mark.parametrize("T", [4096, 8192, 16384, 32768])
 def test_config2_full_size_properties(T):
     """Benchmark config 2 at full size (32 / 8 heads, d_h=128, s96_r4, fp16, one query token):
     split invariance, zero padding rows ignored, agreement with dense fp32 attention on the GPU, 2e-3 bound."""
@@ -238,6 +238,102 @@ def test_argument_checks():
         q.append(cache, x, x, 0)                                                              # capacity exceeded
 
 
+def _two_reference_check(O, Q, cache, xs, lens, what):
+    """Every sequence of a decode batch against two fp32 references computed on the GPU from the cache's own codes
+    (read by tests/helpers.py:unpack_planes, not by the library): attention over the cache decoded with the
+    reference's roundings to the cache dtype (hqmq_attention.py:61-64 of the reference, via dequant_packed) and over
+    the unrounded product.  Bound: tests/helpers.py:assert_attention_close, i.e.
+      |O - exact| <= 2e-3 + 8 * 2^-11 * sum_t p_t |V_t|                (fp16 products, fp32 accumulation)
+      |O - ref_D| <= the same + |ref_D - exact|                        (the reference's own rounding spread).
+    Returns the maxima (|O - exact|, |O - ref_D|, |ref_D - exact|, max |ref_D|)."""
+    from hqmq_amd import ops
+    B = Q.shape[0]
+    T = int(max(lens))
+    Kd_all, Vd_all = ops.dequant_packed(cache.K, T, 0), ops.dequant_packed(cache.V, T, 0)
+    worst = [0.0, 0.0, 0.0, 0.0]
+    for b in range(B):
+        L = int(lens[b])
+        kx, vx = xs(b, L)
+        K_x, V_x = exact_dense(cache.K, b, L, kx), exact_dense(cache.V, b, L, vx)
+        K_D, V_D = Kd_all[b, :, :L].float(), Vd_all[b, :, :L].float()
+        # the library's dense decode and the independent reader agree up to the roundings to the cache dtype
+        eps = 2.0 ** -8 if cache.K.dtype == torch.bfloat16 else 2.0 ** -11
+        assert float(((K_D - K_x).abs() - 3.1 * eps * K_x.abs()).max()) <= 1e-6, f"{what}: K decode of sequence {b}"
+        ref_d, ref_x, a_abs = gpu_attention_refs(Q[b, :, 0], K_D, V_D, K_x, V_x)
+        assert_attention_close(O[b, :, 0], ref_d.cpu(), ref_x.cpu(), a_abs.cpu(), base=2e-3, what=f"{what} sequence {b} (L={L})")
+        got = O[b, :, 0].float()
+        for i, v in enumerate(((got - ref_x).abs().max(), (got - ref_d).abs().max(), (ref_d - ref_x).abs().max(), ref_d.abs().max())):
+            worst[i] = max(worst[i], float(v))
+    print(f"\n{what}: max |O - exact| {worst[0]:.3e}, max |O - ref_D| {worst[1]:.3e}, reference rounding spread "
+          f"max |ref_D - exact| {worst[2]:.3e}, max |ref_D| {worst[3]:.3e}")
+    return worst
+
+
+def test_config4_full_size_properties():
+    """Benchmark config 4 at full size: 32 / 8 heads, d_h 128, batch 64, per-sequence contexts U{1024..16384} (seeded),
+    bf16 activations with lognormal channel scales, s24_r3 + Med3x.  Bulk append, crop to the contexts, one decode
+    step (quantize-and-append of one token per sequence at pos, then attention with kv_lens), checked per sequence
+    against both fp32 references; the batch order and the split count must not change the result."""
+    import hqmq
+    from hqmq_amd import ops
+    dt = torch.bfloat16
+    B, Hq, Hkv, d = 64, 32, 8, 128
+    lens = torch.randint(1024, 16385, (B,), generator=torch.Generator().manual_seed(4)).to(torch.int32)
+    T = int(lens.max()) + 64
+    k = torch.empty(B, Hkv, T, d, dtype=dt, device=DEV)
+    v = torch.empty(B, Hkv, T, d, dtype=dt, device=DEV)
+    g = torch.Generator().manual_seed(44)
+    ck, cv = torch.exp(0.5 * torch.randn(1, Hkv, 1, d, generator=g)), torch.exp(0.5 * torch.randn(1, Hkv, 1, d, generator=g))
+    for b in range(B):                                          # CPU-seeded, one sequence at a time
+        k[b] = (torch.randn(Hkv, T, d, generator=g) * ck[0]).to(dt).to(DEV)
+        v[b] = (torch.randn(Hkv, T, d, generator=g) * cv[0]).to(dt).to(DEV)
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=24, radius_bits=3, device=DEV), C=3.0)
+    cache = w.new_cache(B, T, d, dt, 0, sideband_frac=0.125)
+    w.append(cache, k, v, 0)
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    lens_dev = lens.to(DEV)
+    cache.crop_(lens_dev)
+    # the decode step: one new token per sequence, appended at its own position (its own Med3x statistics: one call)
+    k1 = (torch.randn(B, Hkv, 1, d, generator=g) * ck).to(dt).to(DEV)
+    v1 = (torch.randn(B, Hkv, 1, d, generator=g) * cv).to(dt).to(DEV)
+    pos = lens_dev.clone()
+    w.append(cache, k1, v1, 0, pos=pos)
+    pos += 1
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    Q = torch.randn(B, Hq, 1, d, generator=g).to(dt).to(DEV)
+    order = ops.longest_first(pos)
+    O = hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T, batch_order=order)
+    rate = float(cache.K.sb_count.sum()) / (Hkv * float(pos.sum()) * d / 4)
+    assert 0.002 < rate < 0.05, rate
+
+    def xs(b, L):       # what was quantized into rows [0, L) of sequence b: the bulk rows, then the appended token
+        return (torch.cat([k[b, :, :L - 1], k1[b]], dim=1), torch.cat([v[b, :, :L - 1], v1[b]], dim=1))
+    worst = _two_reference_check(O, Q, cache, xs, pos.cpu().tolist(), "config 4 at full size")
+    assert worst[3] > 0.3                                       # outputs are O(1): the bound is not vacuous
+    # scheduling and splitting do not change the result beyond the merge's fp32 rounding
+    O2 = hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T)
+    assert torch.equal(O2, O)
+    O3 = hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T, n_splits=5, batch_order=order)
+    assert (O3.float() - O.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, worst[3])     # one bf16 ulp of the output
+    Og = hqmq.fused_attention_packed(Q[:4], hqmq.PackedKV(_first(cache.K, 4), _first(cache.V, 4)), kv_lens=pos[:4], T_kv=T,
+                                     force_generic=True)
+    assert (Og.float() - O[:4].float()).abs().max().item() <= 2.0 ** -7 * max(1.0, worst[3])
+
+
+def _first(pt, nb):
+    """A view of the first nb sequences of a PackedTensor (same planes, no copy)."""
+    import copy
+    o = copy.copy(pt)
+    o.B = nb
+    for name in ("main", "aux", "scale", "flags", "sideband", "sb_tile_off", "sb_count", "sb_coord"):
+        t = getattr(pt, name)
+        if t is not None:
+            setattr(o, name, t[:nb])
+    return o
+
+
 @pytest.mark.parametrize("cfg", [3, 5])
 def test_config3_and_5_full_size_properties(cfg):
     """Benchmark configs 3 (28/4 heads, batch 8, 32k, s192_r6 + Med3x, fp16, 2 % of K chunks x50-200) and
@@ -258,14 +354,15 @@ def test_config3_and_5_full_size_properties(cfg):
     w.append(cache, k, v, 0)
     cache.K.check_overflow()
     cache.V.check_overflow()
-    del k, v
     rate = float(cache.K.sb_count.sum()) / (B * Hkv * T * d / 4)
     assert 0.005 < rate < 0.03
     Q = torch.randn(B, Hq, 1, d, generator=torch.Generator().manual_seed(7)).to(dt).to(DEV)
+    O = hqmq.fused_attention_packed(Q, cache)
+    worst = _two_reference_check(O, Q, cache, lambda b, L: (k[b, :, :L], v[b, :, :L]), [T] * B, f"config {cfg} at full size")
+    del k, v
     err, ref_max = dense_check(Q, cache, None, T)
     scale = max(1.0, ref_max)
     assert err < 2e-3 * scale, (err, ref_max)
-    O = hqmq.fused_attention_packed(Q, cache)
     for ns in (1, 5):
         o = hqmq.fused_attention_packed(Q, cache, n_splits=ns)
         assert (o.float() - O.float()).abs().max().item() < 1e-3 * scale
