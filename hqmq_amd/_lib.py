@@ -75,6 +75,7 @@ EXPORTS = [
     "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",
     "hqmq_pack_codes", "hqmq_dequant_packed", "hqmq_attn_workspace_bytes", "hqmq_attn_pick_splits",
     "hqmq_attn_fwd", "hqmq_attn_combine", "hqmq_append_kv", "hqmq_attn_static_scratch_bytes", "hqmq_attn_fwd_static",
+    "hqmq_attn_read_ceiling_sink_bytes", "hqmq_attn_read_ceiling",
 ]
 
 
@@ -91,7 +92,8 @@ def lib():
         L = C.CDLL(str(_SO))
         L.hqmq_status_string.restype = C.c_char_p
         L.hqmq_status_string.argtypes = [C.c_int]
-        for name in ("hqmq_med3x_workspace_bytes", "hqmq_attn_workspace_bytes", "hqmq_attn_static_scratch_bytes"):
+        for name in ("hqmq_med3x_workspace_bytes", "hqmq_attn_workspace_bytes", "hqmq_attn_static_scratch_bytes",
+                     "hqmq_attn_read_ceiling_sink_bytes"):
             getattr(L, name).restype = i64
         _lib = L
     return _lib

@@ -81,7 +81,7 @@ def dense_check(Q, cache, lens, T):
     return worst, ref_max
 
 
-def run(cfg, steps):
+def run(cfg, steps, emit=True):
     if cfg == 3:
         B, Hq, Hkv, d, S, b_r, dt, med = 8, 28, 4, 128, 192, 6, torch.float16, True
         lens, T = None, 32768
@@ -138,8 +138,21 @@ def run(cfg, steps):
     # ragged batch: the longest sequences start first (the order holds while all contexts grow in step)
     order = ops.longest_first(lens_dev) if lens is not None else None
 
+    # a working set below the 256 MB Infinity Cache (config 3: 182 MB) would be served from it on every replay: such a
+    # config alternates between two caches, so that every step reads its cache from HBM as a decode step over many
+    # layers does
+    rot = [cache]
+    if step_bytes < 300e6 and lens is None:
+        k2 = synth(k.shape, dt, 1000 + cfg, outlier_p=0.02 if cfg == 3 else 0.01, gain=(50.0, 200.0) if cfg == 3 else (100.0, 100.0))
+        other = w.new_cache(B, T, d, dt, 0, sideband_frac=0.125)
+        w.append(other, k2, v, 0)
+        rot.append(other)
+        del k2
+    turn = [0]
+
     def attend():
-        hqmq.fused_attention_packed(Q, cache, kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
+        turn[0] += 1
+        hqmq.fused_attention_packed(Q, rot[turn[0] % len(rot)], kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
     us = event_us(attend, steps)
     res = {"config": name, "us_per_step": round(us, 2), "compressed_bytes_per_step": step_bytes,
            "GBps": round(step_bytes / us / 1e3, 1), "pct_of_hbm_roofline": round(100 * step_bytes / us / 1e3 / HBM_PEAK_GBPS, 2),
@@ -174,7 +187,10 @@ def run(cfg, steps):
         res["us_per_step_with_append_graph"] = round(event_us(graph.replay, steps), 2)
         cache.K.check_overflow()
         cache.V.check_overflow()
-    print(json.dumps(res), flush=True)
+    res["caches_rotated"] = len(rot)
+    if emit:
+        print(json.dumps(res), flush=True)
+    return res
 
 
 if __name__ == "__main__":

@@ -297,56 +297,89 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
         if (p.n_splits == 1) {
             store_any(p.O, dtype, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a / l : 0.f);
         } else {
-            float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
+            float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + kPartialHead);
             if (e == 0) { wp[0] = m; wp[1] = l; }
-            wp[2 + e] = a;
+            wp[kPartialHead + e] = a;
         }
     }
 }
 
-// One block per output row, one thread per element.  Every thread loads the (m, l, acc[e]) of up to 32 splits in
-// one batch of independent loads (the m and l of a split are the same addresses in all threads: broadcasts) and
-// merges them in registers, so the kernel costs one round trip to memory per 32 splits; no LDS, no barrier.
-// SC: splits loaded per batch of independent loads (the smallest of 4, 8, 32 that covers n_splits, so that few
-// splits do not pay for 32 predicated loads)
-template <int SC>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
-                                                           int n_splits, int64_t osb, int64_t osh, int64_t ost) {
-    const int64_t row = blockIdx.x;
-    const int e = threadIdx.x;
-    if (e >= d_h) return;
-    const int tq = (int)(row % Tq), hq = (int)((row / Tq) % Hq), b = (int)(row / ((int64_t)Tq * Hq));
-    const float *base = ws + (size_t)row * n_splits * (d_h + 2);
-    float M = -INFINITY, L = 0.f, A = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += SC) {
-        float ms[SC], ls[SC], as[SC];
-#pragma unroll
-        for (int i = 0; i < SC; i++) {
-            const bool ok = s0 + i < n_splits;
-            const float *q = base + (size_t)(ok ? s0 + i : s0) * (d_h + 2);
-            ms[i] = q[0];
-            ls[i] = q[1];
-            as[i] = q[2 + e];
-            if (!ok) { ms[i] = -INFINITY; ls[i] = 0.f; as[i] = 0.f; }
-        }
-        float mx = ms[0];
-#pragma unroll
-        for (int i = 1; i < SC; i++) mx = fmaxf(mx, ms[i]);
-        const float Mn = fmaxf(M, mx);
-        if (Mn > -INFINITY) {
-            const float f = exp2f(M - Mn);       // 0 while M is still -inf
-            L *= f;
-            A *= f;
+// Merge of the split partials: one block of 256 threads per output row.  A thread owns four consecutive output
+// elements (one 16-byte load per split) and every (256 / (d_h / 4))-th split; it loads its splits in batches of four
+// independent (m, l) and acc loads, merges them in registers, and the split groups merge through LDS.  At 32 splits
+// and d_h 128 that is one batch of eight loads per thread: the kernel costs one round trip to memory, one barrier
+// and the launch.
+constexpr int kCombineThreads = 256;
+__global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const float *ws, void *O, int dtype, int Hq, int Tq, int d_h,
+                                                                       int n_splits, int64_t osb, int64_t osh, int64_t ost) {
+    __shared__ float red[kCombineThreads * 6];
+    const unsigned row = blockIdx.x;
+    const int ncol = d_h >> 2, groups = kCombineThreads / ncol;           // d_h <= 256: at least four groups
+    const int c4 = threadIdx.x % ncol, grp = threadIdx.x / ncol;
+    const int rec = d_h + kPartialHead;
+    const float *base = ws + (size_t)row * (size_t)n_splits * rec;
+    float M = -INFINITY, L = 0.f;
+    float4v A = float4v{0.f, 0.f, 0.f, 0.f};
+    if (grp < groups) {
+        constexpr int SC = 4;
+        for (int s0 = grp; s0 < n_splits; s0 += SC * groups) {
+            float2 ml[SC];
+            float4v as[SC];
 #pragma unroll
             for (int i = 0; i < SC; i++) {
-                const float w = exp2f(ms[i] - Mn);
-                L = fmaf(ls[i], w, L);
-                A = fmaf(as[i], w, A);
+                const int s = s0 + i * groups;
+                const float *q = base + (size_t)min(s, n_splits - 1) * rec;
+                ml[i] = *reinterpret_cast<const float2 *>(q);
+                as[i] = *reinterpret_cast<const float4v *>(q + kPartialHead + 4 * c4);
+                if (s >= n_splits) { ml[i] = float2{-INFINITY, 0.f}; as[i] = float4v{0.f, 0.f, 0.f, 0.f}; }
             }
-            M = Mn;
+            float mx = M;
+#pragma unroll
+            for (int i = 0; i < SC; i++) mx = fmaxf(mx, ml[i].x);
+            if (mx > -INFINITY) {
+                const float f = exp2f(M - mx);          // 0 while M is still -inf
+                L *= f;
+                A = A * f;
+#pragma unroll
+                for (int i = 0; i < SC; i++) {
+                    const float w = exp2f(ml[i].x - mx);
+                    L = fmaf(ml[i].y, w, L);
+                    A = A + as[i] * w;
+                }
+                M = mx;
+            }
+        }
+        float *r = red + (size_t)threadIdx.x * 6;
+        r[0] = M; r[1] = L; r[2] = A[0]; r[3] = A[1]; r[4] = A[2]; r[5] = A[3];
+    }
+    __syncthreads();
+    if (grp != 0) return;
+    for (int g = 1; g < groups; g++) {
+        const float *r = red + (size_t)(g * ncol + c4) * 6;
+        const float m2 = r[0];
+        const float mx = fmaxf(M, m2);
+        if (mx > -INFINITY) {
+            const float f = exp2f(M - mx), w = exp2f(m2 - mx);
+            L = fmaf(r[1], w, L * f);
+            A = A * f + float4v{r[2], r[3], r[4], r[5]} * w;
+            M = mx;
         }
     }
-    store_any(O, dtype, b * osb + hq * osh + (int64_t)tq * ost + e, L > 0.f ? A / L : 0.f);
+    const unsigned bh = row / (unsigned)Tq, tq = row - bh * (unsigned)Tq, b = bh / (unsigned)Hq, hq = bh - b * (unsigned)Hq;
+    const int64_t o = (int64_t)b * osb + (int64_t)hq * osh + (int64_t)tq * ost + 4 * c4;
+    float r[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = L > 0.f ? A[e] / L : 0.f;
+    if (dtype != HQMQ_F32 && ((((uintptr_t)O) | (uintptr_t)(osb * 2) | (uintptr_t)(osh * 2) | (uintptr_t)(ost * 2)) & 7) == 0) {
+        // four 16-bit results as one 8-byte store
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = dtype == HQMQ_F16 ? __half_as_ushort(__float2half_rn(r[e])) : f32_to_bf16_bits(r[e]);
+        *reinterpret_cast<uint2 *>((uint16_t *)O + o) = uint2{(uint32_t)h[0] | (uint32_t)h[1] << 16, (uint32_t)h[2] | (uint32_t)h[3] << 16};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) store_any(O, dtype, o + e, r[e]);
+    }
 }
 
 static PackedDev to_dev(const hqmq_packed &k) {
@@ -383,7 +416,7 @@ using namespace hqmq;
 
 extern "C" int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits) {
     if (n_splits <= 1) return 0;
-    return (int64_t)B * H_q * T_q * n_splits * (d_h + 2) * 4;
+    return (int64_t)B * H_q * T_q * n_splits * (d_h + kPartialHead) * 4;
 }
 
 // Blocks per (sequence, KV head, column group): one block per CU, each of a block's eight wavefronts
@@ -409,10 +442,9 @@ extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int 
     if (dtype != HQMQ_F32 && dtype != HQMQ_F16 && dtype != HQMQ_BF16) return HQMQ_ERR_DTYPE;
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
-    auto kern = n_splits <= 4 ? attn_combine_kernel<4> : n_splits <= 8 ? attn_combine_kernel<8> : attn_combine_kernel<32>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3((d_h + 63) / 64 * 64), 0, (hipStream_t)stream,
-                       (const float *)workspace, O,
-                       dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
+    if ((uintptr_t)workspace & 15) return HQMQ_ERR_ALIGN;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(kCombineThreads), 0, (hipStream_t)stream,
+                       (const float *)workspace, O, dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
 }
 
@@ -448,7 +480,7 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     if (n_splits > 1) {
         if (!a->workspace) return HQMQ_ERR_NULL;
         if (a->workspace_bytes < hqmq_attn_workspace_bytes(a->B, a->H_q, a->T_q, 4 * n, n_splits)) return HQMQ_ERR_WORKSPACE;
-        if ((uintptr_t)a->workspace & 3) return HQMQ_ERR_ALIGN;
+        if ((uintptr_t)a->workspace & 15) return HQMQ_ERR_ALIGN;
     }
     // LDS: the two fp16 codeword tables, reused afterwards for the cross-wave merge
     size_t shmem = ((size_t)a->K.K + a->V.K) * 8;

@@ -10,6 +10,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 
 constexpr int kAttnWaves = 4;
 constexpr int kSuper = 64;  // tokens per super-tile
+constexpr int kPartialHead = 4;  // floats in front of the accumulators of a split partial (m, l, 2 unused): keeps acc 16-byte aligned
 
 struct PackedDev {
     const uint8_t *main_plane, *aux_plane, *flag_plane;
@@ -44,7 +45,7 @@ struct AttnParams {
     float inv_qmax;
     int n_splits, n_cg;
     int scale_vec;  // scales of 4 consecutive tokens may be read with one aligned vector load
-    float *ws;      // split partials [row][split][d_h + 2]
+    float *ws;      // split partials [row][split][kPartialHead + d_h]: m (base-2 exponent units), l, two unused floats, acc
     int xcd_remap;  // blocks of one (sequence, KV head) share an XCD (see attn_fast_kernel)
 };
 

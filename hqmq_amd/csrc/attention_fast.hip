@@ -168,14 +168,17 @@ __device__ __forceinline__ uint32_t half_addr8(uint32_t pair) {
     return r;
 }
 
-// Decodes the CPL chunks of one lane: gather from the LDS table, times the radius code.
+// Decode of the CPL chunks of one lane in two steps, so that a caller can put all gathers of a half-step in flight
+// before the first multiply: gather_chunks requests the codewords from the LDS table (g) and prepares the radius
+// codes as packed fp16 pairs (r, chunk j in r[j / 2][j & 1]); scale_chunks multiplies.
 // 16+0 layout: the two radius codes of a dword become an fp16 pair with one shift, one and-or
 // (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract.  IB = idx_bits when known at compile
 // time (12 for s96), else 0.
 template <int CPL, int MB, int AB, int IB, int NW, int TAB_OFF>
-__device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t aux, int idx_bits_rt, half4 (&a)[CPL]) {
+__device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t aux, int idx_bits_rt, half4 (&g)[CPL], half2v (&r)[CPL / 2]) {
     const int idx_bits = IB ? IB : idx_bits_rt;
     const uint32_t idx_mask = (1u << idx_bits) - 1u;
+    const half2v k1024 = half2v{(_Float16)1024.0f, (_Float16)1024.0f};
     if constexpr (MB == 16 && AB == 0) {
         // mask in a scalar register and magic in a vector register, so that (x & mask) | magic is one v_and_or_b32
         uint32_t rq2 = (0xffffu >> idx_bits) * 0x00010001u, magic = 0x64006400u;
@@ -185,10 +188,10 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
+            g[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix));
+            g[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix));
             const uint32_t t = ((w[i] >> idx_bits) & rq2) | magic;
-            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix)) * r[0];
-            a[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix)) * r[1];
+            r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
     } else if constexpr (MB == 16 && AB == 3 && IB == 13) {
         // s192_r6: idx (13 bits) and the low three radius bits in the 16-bit main field, the high three in the aux
@@ -198,11 +201,11 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
+            g[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix));
+            g[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix));
             const uint32_t hi = *(lds_u1_ptr)(uintptr_t)(kAuxTabOffset + ((aux >> (6 * i)) & 63u) * 4u);
             const uint32_t t = ((w[i] >> 13) & 0x00070007u) | hi;
-            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix)) * r[0];
-            a[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix)) * r[1];
+            r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
     } else if constexpr (MB == 12 && AB == 1 && IB == 10 && CPL == 8) {
         // s24_r3: eight 12-bit fields (idx in the low 10 bits, the low two radius bits above) in three dwords
@@ -214,25 +217,30 @@ __device__ __forceinline__ void decode_chunks(const uint32_t (&w)[NW], uint32_t 
         constexpr uint32_t M = 0x1ff8u;
         const uint32_t ad[8] = {(w0 << 3) & M, (w0 >> 9) & M, __builtin_amdgcn_alignbit(w1, w0, 21) & M, (w1 >> 1) & M,
                                 (w1 >> 13) & M, __builtin_amdgcn_alignbit(w2, w1, 25) & M, (w2 >> 5) & M, (w2 >> 17) & M};
+#pragma unroll
+        for (int j = 0; j < 8; j++) g[j] = gather8<TAB_OFF>(ad[j]);
         const uint32_t lo2[8] = {__builtin_amdgcn_ubfe(w0, 10, 2), __builtin_amdgcn_ubfe(w0, 22, 2), __builtin_amdgcn_ubfe(w1, 2, 2),
                                  __builtin_amdgcn_ubfe(w1, 14, 2), __builtin_amdgcn_ubfe(w1, 26, 2), __builtin_amdgcn_ubfe(w2, 6, 2),
                                  __builtin_amdgcn_ubfe(w2, 18, 2), w2 >> 30};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t t = (lo2[2 * i] | (lo2[2 * i + 1] << 16)) | axs[i];
-            const half2v r = __builtin_bit_cast(half2v, t) - half2v{(_Float16)1024.0f, (_Float16)1024.0f};
-            a[2 * i] = gather8<TAB_OFF>(ad[2 * i]) * r[0];
-            a[2 * i + 1] = gather8<TAB_OFF>(ad[2 * i + 1]) * r[1];
+            r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
     } else {
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             uint32_t code = code_at<MB, NW>(w, j);
             if (AB) code |= ((aux >> (j * AB)) & ((1u << AB) - 1u)) << MB;
-            const _Float16 rq = (_Float16)(uint16_t)(code >> idx_bits);
-            a[j] = gather8<TAB_OFF>((code & idx_mask) << 3) * rq;
+            g[j] = gather8<TAB_OFF>((code & idx_mask) << 3);
+            r[j >> 1][j & 1] = (_Float16)(uint16_t)(code >> idx_bits);
         }
     }
+}
+template <int CPL>
+__device__ __forceinline__ void scale_chunks(const half4 (&g)[CPL], const half2v (&r)[CPL / 2], half4 (&a)[CPL]) {
+#pragma unroll
+    for (int j = 0; j < CPL; j++) a[j] = g[j] * r[j >> 1][j & 1];
 }
 
 __device__ __forceinline__ half8 cat8(half4 x, half4 y) { return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7); }
@@ -274,6 +282,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     static_assert(CPL % 2 == 0, "two chunks per 16x16x32 operand");
     constexpr int NT = WV * 64;
     constexpr int kKPre = CPL >= 8 ? 3 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
+    constexpr bool kBatchGathers = false;       // see half_step: measured, no gain on any shape (178 against 157 registers)
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
@@ -390,12 +399,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[cgi] * p.qsh + (int64_t)tq[cgi] * p.qst + grp * CPL * 4;
 #pragma unroll
         for (int j = 0; j < CPL / 2; j++) {
-            // columns out of range point at a valid row (tq = 0, first head of the group): load, then clear
-            // (an and with a lane mask, not a conditional: no branch and no wait between the loads)
-            const uint32_t keep = col_ok[cgi] ? 0xffffffffu : 0u;
-            uint2 lo = *reinterpret_cast<const uint2 *>(qp + 8 * j), hi = *reinterpret_cast<const uint2 *>(qp + 8 * j + 4);
-            lo.x &= keep; lo.y &= keep; hi.x &= keep; hi.y &= keep;
-            qf[cgi][j] = cat8(chunk_to_half<DT>(lo), chunk_to_half<DT>(hi));
+            // only the lanes of real columns load (a decode step has G of 16): masked-off lanes cost the memory
+            // pipeline nothing, a clamped load would cost it a full request
+            const half4 z = half4{0, 0, 0, 0};
+            const half4 lo = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
+            const half4 hi = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
+            qf[cgi][j] = cat8(lo, hi);
         }
     }
     auto load_flags = [&](int th, FlagTile &f) {
@@ -642,10 +651,21 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre<kKPre> &kc, const VPre<kVPre> &vc) {
         float4v sT[NCG][2], so[2] = {zero4, zero4};
         if (FLAGS) k_apply(kc, so);
+        // every gather of the 32 K tokens is requested before the first one is used: the wavefront waits for LDS
+        // once per half-step and tensor, not once per pair of chunks
+        // (the variants that have no registers to spare keep the compiler's own interleaving of gathers and multiplies)
+        half4 gk[2][CPL];
+        half2v rk[2][CPL / 2];
+        if constexpr (kBatchGathers) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
-            decode_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, a);
+            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
+            scale_chunks<CPL>(gk[u], rk[u], a);
 #pragma unroll
             for (int cgi = 0; cgi < NCG; cgi++) {
                 float4v s = zero4;
@@ -657,6 +677,14 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                     s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[u][e] * qmaxf : 0.f);
                 sT[cgi][u] = s;
             }
+        }
+        // the V gathers fly while the softmax below keeps the vector unit busy
+        half4 gv[2][CPL];
+        half2v rv[2][CPL / 2];
+        if constexpr (kBatchGathers) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         // ---- mask (boundary half-steps only), online softmax, per column group ----
         const bool edge = !(th + 32 <= lim_min && th + 32 <= t_end && th >= col_start);
@@ -704,10 +732,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             pp[cgi] = cat8(pT[0], pT[1]);
         }
         // ---- O^T += V^T . P^T, both tiles in one MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
+        if constexpr (kBatchGathers) __builtin_amdgcn_sched_barrier(0);
         half4 av[2][CPL];
 #pragma unroll
-        for (int u = 0; u < 2; u++)
-            decode_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, av[u]);
+        for (int u = 0; u < 2; u++) {
+            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            scale_chunks<CPL>(gv[u], rv[u], av[u]);
+        }
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
@@ -814,9 +845,9 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
             } else {
                 // partials carry the maximum in softmax units (base-2 exponent) and acc already divided by qmax
-                float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + 2);
+                float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + kPartialHead);
                 if (e == 0) { wp[0] = m * c; wp[1] = l; }
-                wp[2 + e] = a * inv_qmax;
+                wp[kPartialHead + e] = a * inv_qmax;
             }
         }
     }

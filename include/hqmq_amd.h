@@ -195,7 +195,7 @@ int hqmq_dequant_packed(const hqmq_packed *p, int dtype, int B, int H, int T, in
  * Query row i of sequence b sees key j iff j < kv_len[b] (T_kv when kv_len is
  * NULL) and (not causal or j <= i + causal_offset); causal_offset = 0 is the
  * reference's top-left alignment.
- *   workspace   hqmq_attn_workspace_bytes(...) bytes of scratch for split-KV partials, any content */
+ *   workspace   hqmq_attn_workspace_bytes(...) bytes of scratch for split-KV partials, 16-byte aligned, any content */
 typedef struct hqmq_attn_args {
     const void *Q; void *O;   /* D, [B][H_q][T_q][d_h]; strides in elements, last dim contiguous */
     int64_t q_sb, q_sh, q_st, o_sb, o_sh, o_st;
@@ -239,6 +239,17 @@ int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q,
 #define HQMQ_ATTN_STATIC_SCRATCH_BYTES (8 << 20)
 int64_t hqmq_attn_static_scratch_bytes(void);
 int hqmq_attn_fwd_static(const hqmq_attn_args *a, void *stream);
+
+/* Measurement aid, no counterpart in the reference: a kernel that only reads the K and V planes of a packed cache
+ * with the grid, the per-wavefront token ranges and the per-lane loads of the specialised decode-attention kernel
+ * (16+0 layout at d_h = 128, no sideband; other layouts return HQMQ_ERR_LAYOUT).  Its duration is the time the
+ * memory system needs for a launch of this shape; bench.py reports it beside the attention kernel's.
+ *   a       as for hqmq_attn_fwd (Q, O, tables and workspace are not touched; start_event / stop_event are honoured)
+ *   depth   32-token steps per wavefront in the ring: depth - 1 are in flight (2, 3, 4 or 6; the attention kernel uses 3)
+ *   waves   wavefronts per block, 8 or 12
+ *   sink    hqmq_attn_read_ceiling_sink_bytes(B, H_kv, n_splits) bytes that receive one word per thread */
+int64_t hqmq_attn_read_ceiling_sink_bytes(int B, int H_kv, int n_splits);
+int hqmq_attn_read_ceiling(const hqmq_attn_args *a, int depth, int waves, void *sink, int64_t sink_bytes, void *stream);
 
 #ifdef __cplusplus
 }
