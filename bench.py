@@ -263,9 +263,12 @@ def main():
     value = step_bytes / (us_step * 1e-6) / 1e9
 
     # the attention kernel alone (split partials left in the workspace), a pair of HIP events per launch
+    partials = torch.empty(max(16, int(ops.L.lib().hqmq_attn_workspace_bytes(1, Hq, 1, D_H, n_splits))), dtype=torch.uint8, device=dev)
+
     def main_kernel(i, ev, rotate=True):
         j = i % NL if rotate else 0
-        ops.attn_fwd(queries[j], caches[j].K, caches[j].V, T, n_splits=n_splits, out=outs[j], skip_combine=True, kernel_events=ev)
+        ops.attn_fwd(queries[j], caches[j].K, caches[j].V, T, n_splits=n_splits, out=outs[j], skip_combine=True, kernel_events=ev,
+                     workspace=partials)
     us_main = kernel_time_us(main_kernel, 192)
     us_main_same = kernel_time_us(lambda i, ev: main_kernel(i, ev, False), 192)
     us_launch_interval, _ = graph_us(lambda i: main_kernel(i, None), args.steps, stream)

@@ -34,7 +34,7 @@ class QuantizeArgs(C.Structure):
         ("thr", vp), ("mask_out", vp),
         ("main_plane", vp), ("aux_plane", vp), ("flag_plane", vp), ("scale_plane", vp),
         ("t_cap", i64), ("t_off", C.c_int), ("pos", vp), ("main_bits", C.c_int), ("aux_bits", C.c_int),
-        ("stats", vp),
+        ("stats", vp), ("scale_max_bits", vp),
     ]
 
 
@@ -52,7 +52,7 @@ class Packed(C.Structure):
         ("main_plane", vp), ("aux_plane", vp), ("flag_plane", vp), ("scale_plane", vp),
         ("scale_sb", i64), ("scale_sh", i64), ("scale_st", i64),
         ("sideband", vp), ("sb_tile_off", vp), ("sb_cap", i64), ("sb_coord", vp), ("sb_count", vp),
-        ("joint", vp), ("joint_sh", i64), ("K", C.c_int),
+        ("joint", vp), ("joint_sh", i64), ("K", C.c_int), ("scale_max_bits", vp),
     ]
 
 

@@ -52,6 +52,8 @@ def _pack_unpacked(idx, rq, rs, joint, r_qmax: int) -> PackedTensor:
     pt.qmax = int(r_qmax)
     ops.pack_codes(idx, rq, pt)
     pt.scale[:, :, :T] = rs            # into the padded plane: rows up to the capacity stay readable
+    if pt.scale_max is not None:       # the range guard of bf16 / fp32 caches: the largest finite scale, as fp32 bits
+        pt.scale_max = torch.nan_to_num(rs.detach().float().abs(), nan=0.0, posinf=0.0).amax().reshape(1).view(torch.int32)
     pt.length = T
     return pt
 

@@ -148,6 +148,11 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
     float4v acc[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    // Range guard of bf16 / fp32 caches (see attention_common.h): the softmax weights carry 2^-eshift, so that
+    // P * (V scale) fits fp16; verbatim outlier chunks are brought into range by the same bounds (a verbatim value
+    // never exceeds its token's scale) and meet the weights without the offset (V) or are rescaled in fp32 (K).
+    const float eshift = v_scale_shift(p.Vc), kshift = FLAGS ? v_scale_shift(p.Kc) : 0.f;
+    const float v_down = exp2f(-eshift), p_up = exp2f(eshift), k_down = exp2f(-kshift), k_up = exp2f(kshift) * p.c_plain;
 
     for (int t0 = t_begin; t0 < t_end; t0 += kSuper) {
         SuperTile<NW> nxt;
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
                     if (__builtin_amdgcn_ballot_w64(f) != 0) {
                         half4 ao = half4{0, 0, 0, 0};
                         if (f) {
-                            ao = outlier_chunk(p.Kc, dtype, bh, sb_base + __popc(fl & ((1u << j) - 1u)));
+                            ao = outlier_chunk(p.Kc, dtype, bh, sb_base + __popc(fl & ((1u << j) - 1u)), k_down);
                             a = half4{0, 0, 0, 0};
                         }
                         so = __builtin_amdgcn_mfma_f32_16x16x16f16(ao, qf[j], so, 0, 0, 0);
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + 16 * u + 4 * grp + e;
                 float v = sT[u][e] * (cur.ks[u][e] * p.c_log2);
-                if (FLAGS) v = fmaf(sTo[u][e], p.c_plain, v);
+                if (FLAGS) v = fmaf(sTo[u][e], k_up, v);
                 v = (t < col_lim && t < t_end && t >= col_start) ? v : -INFINITY;
                 pv[u][e] = v;
                 tmax = fmaxf(tmax, v);
@@ -218,10 +223,10 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
         for (int u = 0; u < 4; u++) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const float pe = exp2f(pv[u][e] - m_use);
+                const float pe = exp2f(pv[u][e] - m_use - eshift);
                 l_run += pe;
                 pT[u][e] = (_Float16)(pe * (cur.vs[u][e] * p.inv_qmax));
-                if (FLAGS) pTo[u][e] = (_Float16)pe;
+                if (FLAGS) pTo[u][e] = (_Float16)(pe * p_up);          // without the offset: at most 1
             }
         }
         // ---------------- O^T += V^T . P^T ----------------
@@ -245,7 +250,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_kernel(AttnParams p) {
                     if (__builtin_amdgcn_ballot_w64(f) != 0) {
                         half4 ao = half4{0, 0, 0, 0};
                         if (f) {
-                            ao = outlier_chunk(p.Vc, dtype, bh, sb_base + __popc(fl & ((1u << j) - 1u)));
+                            ao = outlier_chunk(p.Vc, dtype, bh, sb_base + __popc(fl & ((1u << j) - 1u)), v_down);
                             a = half4{0, 0, 0, 0};
                         }
                         uint2 ro = __builtin_bit_cast(uint2, ao);
@@ -384,7 +389,7 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const flo
 
 static PackedDev to_dev(const hqmq_packed &k) {
     return PackedDev{k.main_plane, k.aux_plane, k.flag_plane, k.scale_plane, k.scale_sb, k.scale_sh, k.scale_st,
-                     k.sideband, k.sb_tile_off, k.sb_cap, k.sb_coord, k.sb_count, k.joint, k.joint_sh, k.K};
+                     k.sideband, k.sb_tile_off, k.sb_cap, k.sb_coord, k.sb_count, k.joint, k.joint_sh, k.K, k.scale_max_bits};
 }
 
 template <int CPL, int MB>

@@ -24,6 +24,7 @@ struct PackedDev {
     const void *joint;
     int64_t jsh;
     int K;
+    const uint32_t *scale_max;
 };
 
 struct AttnParams {
@@ -162,12 +163,18 @@ __device__ __forceinline__ void tile_flags(const PackedDev &c, size_t plane_row0
     slot0 = max(tile_off, 0) + pre_t + __popc(fw_t & ((first >= 32) ? 0xffffffffu : ((1u << first) - 1u)));
 }
 
-// A flagged chunk: the verbatim values from the sideband (exact in fp16 for fp16 caches).
-__device__ __forceinline__ half4 outlier_chunk(const PackedDev &c, int dtype, size_t bh, int slot) {
+// A flagged chunk: the verbatim values from the sideband (exact in fp16 for fp16 caches), times `down`: 1, or the
+// power of two that brings a bf16 / fp32 cache whose values leave the fp16 range back into it (a verbatim value is
+// bounded by its token's scale, so the bound of the scales serves).
+__device__ __forceinline__ half4 outlier_chunk(const PackedDev &c, int dtype, size_t bh, int slot, float down) {
     int64_t s = slot;
     if (s >= c.sb_cap) s = c.sb_cap - 1;
     if (s < 0) s = 0;
-    return load_chunk_h(c.sideband, dtype, (int64_t)bh * c.sb_cap + s);
+    const int64_t chunk = (int64_t)bh * c.sb_cap + s;
+    if (dtype == HQMQ_F16) return load_chunk_h(c.sideband, dtype, chunk);
+    half4 r;
+    for (int j = 0; j < 4; j++) r[j] = (_Float16)(load_any(c.sideband, dtype, chunk * 4 + j) * down);
+    return r;
 }
 
 
@@ -189,6 +196,15 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
             if (k < K) dst[k] = __builtin_bit_cast(uint2, tmp[u]);
         }
     }
+}
+
+// Power-of-two offset of the softmax exponent that keeps P * (V scale) inside fp16: 0 while the largest V scale is
+// below 2^15, else its excess exponent.  Numerator and denominator of the attention output carry the same factor.
+__device__ __forceinline__ float v_scale_shift(const PackedDev &v) {
+    if (!v.scale_max) return 0.f;
+    const uint32_t bits = __builtin_nontemporal_load(v.scale_max);
+    const int e = (int)((bits >> 23) & 0xffu) - 127 + 1;        // scale < 2^e
+    return (float)max(e - 15, 0);
 }
 
 // Implemented in attention_fast.hip: kernels specialised at compile time for the common layouts

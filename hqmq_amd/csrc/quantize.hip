@@ -50,6 +50,7 @@ struct QParams {
     int idx_bits, main_bits, aux_bits;
     int tokens_per_block;
     int32_t *stats;
+    uint32_t *scale_max;
     // sideband compaction in the same launch (compact != 0): see the end of quantize_body
     int compact;
     void *sideband;
@@ -422,6 +423,14 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             }
             if (a.scale_plane && c == 0) D::store((ST *)a.scale_plane + prow, rm);
         }
+        if (a.scale_max && a.scale_plane) {
+            // the largest finite scale written so far, for the attention kernels' range guard: the wavefront's maximum,
+            // and an atomic only when it raises the value (after the first blocks it hardly ever does)
+            uint32_t mine = (row_ok && c == 0 && rm < INFINITY) ? __float_as_uint(rm) : 0u;     // scales are positive: bits order like values
+            for (int o = 1; o < 64; o <<= 1) mine = max(mine, (uint32_t)__shfl_xor((int)mine, o, 64));
+            if ((tid & 63) == 0 && mine > __hip_atomic_load(a.scale_max, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                atomicMax(a.scale_max, mine);
+        }
         if (a.compact) {
             // Sideband compaction in the same launch, for appends whose new rows of a (b, h) all sit in this block
             // (T <= tokens_per_block; n a power of two, so the lanes of a token share a wavefront).  Entries, tile
@@ -559,6 +568,7 @@ static int fill_qparams(const hqmq_quantize_args *a, QParams *out, bool *empty) 
     p.idx_bits = ib; p.main_bits = packed ? a->main_bits : mb; p.aux_bits = packed ? a->aux_bits : ab;
     p.tokens_per_block = kQThreads / a->n_chunks;
     p.stats = a->stats;
+    p.scale_max = a->scale_max_bits;
     p.compact = 0;
     p.sideband = nullptr; p.sb_cap = 0; p.sb_tile_off = p.sb_count = p.overflow = nullptr; p.sb_coord = nullptr;
     return HQMQ_OK;

@@ -48,11 +48,16 @@ class QuantizedCache(DynamicCache):
 class PackedLayer(DynamicLayer):
     """One layer's compressed K and V."""
 
-    def __init__(self, quantizer, layer_idx: int, max_tokens: int, sideband_frac: float):
+    def __init__(self, quantizer, layer_idx: int, max_tokens: int, sideband_frac: float, overflow_check_every: int = 256):
         super().__init__()
         self.quantizer, self.layer_idx, self.max_tokens, self.sideband_frac = quantizer, layer_idx, max_tokens, sideband_frac
         self.packed = None
         self.n_tokens = 0
+        # a sideband that runs full drops outlier chunks (they then decode to zero): the flag the kernels set is read
+        # back after the first append (the prefill) and then once every `overflow_check_every` appends (one device
+        # read each time; 0 = never, call check_overflow() yourself)
+        self.overflow_check_every = overflow_check_every
+        self._appends = 0
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, *args, **kwargs):
         if self.packed is None:
@@ -66,6 +71,11 @@ class PackedLayer(DynamicLayer):
             raise HqmqError(f"PackedQuantizedCache holds {self.packed.K.t_cap} tokens per sequence; raise max_tokens")
         self.quantizer.append(self.packed, key_states, value_states, self.layer_idx)
         self.n_tokens += key_states.shape[2]
+        self._appends += 1
+        if self.packed.K.has_outliers and self.overflow_check_every and (
+                self._appends == 1 or self._appends % self.overflow_check_every == 0):
+            self.packed.K.check_overflow()
+            self.packed.V.check_overflow()
         key_states.hqmq_layer = self          # how hqmq_packed_attention finds the planes
         return key_states, value_states
 
@@ -96,15 +106,17 @@ class PackedLayer(DynamicLayer):
 class PackedQuantizedCache(DynamicCache):
     """Keeps every layer bit-packed; use with attn_implementation="hqmq_packed"."""
 
-    def __init__(self, quantizer, max_tokens: int, sideband_frac: float = 0.125):
+    def __init__(self, quantizer, max_tokens: int, sideband_frac: float = 0.125, overflow_check_every: int = 256):
         super().__init__()
         if not hasattr(quantizer, "append") or not hasattr(quantizer, "new_cache"):
             raise TypeError("PackedQuantizedCache needs an HQMQ quantizer (HQMQ(...) or with_outlier_extraction(HQMQ(...)))")
         self.quantizer, self.max_tokens, self.sideband_frac = quantizer, int(max_tokens), sideband_frac
+        self.overflow_check_every = overflow_check_every
 
     def update(self, key_states, value_states, layer_idx, *args, **kwargs):
         while len(self.layers) <= layer_idx:
-            self.layers.append(PackedLayer(self.quantizer, len(self.layers), self.max_tokens, self.sideband_frac))
+            self.layers.append(PackedLayer(self.quantizer, len(self.layers), self.max_tokens, self.sideband_frac,
+                                           self.overflow_check_every))
         return self.layers[layer_idx].update(key_states, value_states, *args, **kwargs)
 
     def check_overflow(self) -> None:

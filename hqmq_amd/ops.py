@@ -91,6 +91,7 @@ def quantize(x: torch.Tensor, joint: torch.Tensor, slack: Optional[torch.Tensor]
         a.flag_plane = L.ptr(cache.flags) if thr is not None else None
         a.t_cap, a.t_off = cache.t_cap, t_off
         a.main_bits, a.aux_bits = cache.main_bits, cache.aux_bits
+        a.scale_max_bits = L.ptr(cache.scale_max)
         if pos is not None:
             pos = pos.to(device=dev, dtype=torch.int32).contiguous()
             keep.append(pos)
@@ -106,24 +107,40 @@ def quantize(x: torch.Tensor, joint: torch.Tensor, slack: Optional[torch.Tensor]
 
 _WS = {}
 
+# torch.quantile refuses more than 2^24 elements along the reduced dimension ("quantile() input tensor is too large"),
+# which bounds the chunks per head of one Med-C call of the reference (src/quantizers/outlier_aware.py:68).  The
+# radix select here has no such bound; check_quantile_limit(..., strict=True) mirrors the reference's refusal.
+QUANTILE_LIMIT = 1 << 24
+
+
+def check_quantile_limit(chunks_per_head: int, strict: bool) -> bool:
+    """True when a Med-C call of this size is within torch.quantile's limit.  Beyond it the reference raises; with
+    strict=True so does this function (same exception type and message), otherwise the call is an extension."""
+    ok = chunks_per_head <= QUANTILE_LIMIT
+    if not ok and strict:
+        raise RuntimeError("quantile() input tensor is too large")
+    return ok
+
 
 def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
-    """A cached scratch buffer of at least nbytes (grown on demand, reused across calls)."""
+    """A cached scratch buffer of at least nbytes (grown on demand, reused across calls on the same stream; any content)."""
     dev = torch.device(device)
     key = (tag, dev, torch.cuda.current_stream(dev).cuda_stream)     # calls on different streams may overlap
     buf = _WS.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)   # attention counters start at zero
+        buf = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
         _WS[key] = buf
     return buf
 
 
-def med3x_threshold(x: torch.Tensor, mult: float = 3.0, want_count: bool = True):
-    """Per-head (median fp32, threshold in x.dtype, #chunks above threshold int32) over the whole call."""
+def med3x_threshold(x: torch.Tensor, mult: float = 3.0, want_count: bool = True, strict_quantile_limit: bool = False):
+    """Per-head (median fp32, threshold in x.dtype, #chunks above threshold int32) over the whole call.
+    strict_quantile_limit: raise as the reference does when a head has more than 2^24 chunks in this call."""
     L.require_gpu(x, "x")
     x = _strided_x(x)
     B, H, T, d_h = x.shape
     n = d_h // 4
+    check_quantile_limit(B * T * n, strict_quantile_limit)
     dev = x.device
     nbytes = int(L.lib().hqmq_med3x_workspace_bytes(C.c_int(H), C.c_int(_dt(x))))
     ws = _workspace(nbytes, dev, "med3x")
@@ -200,6 +217,7 @@ def append_kv(k: torch.Tensor, v: torch.Tensor, k_cache, v_cache, k_joint, k_sla
         q.main_plane, q.aux_plane, q.scale_plane = L.ptr(cache.main), L.ptr(cache.aux), L.ptr(cache.scale)
         q.t_cap, q.t_off = cache.t_cap, t_off
         q.main_bits, q.aux_bits = cache.main_bits, cache.aux_bits
+        q.scale_max_bits = L.ptr(cache.scale_max)
         q.pos = L.ptr(pos)
         keep += [x, joint, slack]
         cnt = None
@@ -291,12 +309,15 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
              force_generic: bool = False, kernel_events: Optional[tuple] = None,
-             static_scratch: bool = False) -> torch.Tensor:
+             static_scratch: bool = False, workspace: Optional[torch.Tensor] = None):
     """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each).
     kernel_events: two raw hipEvent_t handles (ints) that receive the GPU timestamps of the begin and the end of
     the main attention kernel (profiling).
     static_scratch: call hqmq_attn_fwd_static, which keeps the split partials in the library's own device array
-    instead of a torch workspace (pass `out` as well and the call allocates nothing on the device)."""
+    instead of a torch workspace (pass `out` as well and the call allocates nothing on the device).
+    skip_combine: leave the split partials unmerged and return (O, partials, n_splits): the partials are in `workspace`
+    if given, else in a buffer of their own (never the cached scratch that the next call on the stream overwrites);
+    attn_combine(partials, O, n_splits) merges them."""
     L.require_gpu(Q, "Q")
     if Q.stride(-1) != 1:
         Q = Q.contiguous()
@@ -351,10 +372,31 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
         return O
     if n_splits > 1:
         nbytes = int(L.lib().hqmq_attn_workspace_bytes(C.c_int(B), C.c_int(Hq), C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits)))
-        ws = _workspace(nbytes, dev, "attn")
-        a.workspace, a.workspace_bytes = L.ptr(ws), ws.numel()
+        if workspace is not None:
+            if workspace.device != dev or workspace.numel() * workspace.element_size() < nbytes:
+                raise L.HqmqError(f"workspace must hold {nbytes} bytes on {dev}")
+            ws = workspace
+        elif skip_combine:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        else:
+            ws = _workspace(nbytes, dev, "attn")
+        a.workspace, a.workspace_bytes = L.ptr(ws), ws.numel() * ws.element_size()
     with torch.cuda.device(dev):
         L.check(L.lib().hqmq_attn_fwd(C.byref(a), L.stream_ptr(dev)), "hqmq_attn_fwd")
+    if skip_combine:
+        return O, ws, n_splits
+    return O
+
+
+def attn_combine(partials: Optional[torch.Tensor], O: torch.Tensor, n_splits: int) -> torch.Tensor:
+    """Merge the split partials a skip_combine call left behind into O (B, H_q, T_q, d_h)."""
+    if n_splits <= 1 or partials is None:
+        return O
+    B, Hq, Tq, d_h = O.shape
+    with torch.cuda.device(O.device):
+        L.check(L.lib().hqmq_attn_combine(L.ptr(partials), L.ptr(O), C.c_int(L.DT_CODE[O.dtype]), C.c_int(B), C.c_int(Hq),
+                                          C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits), L.i64(O.stride(0)), L.i64(O.stride(1)),
+                                          L.i64(O.stride(2)), L.stream_ptr(O.device)), "hqmq_attn_combine")
     return O
 
 

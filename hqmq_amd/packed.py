@@ -44,6 +44,9 @@ class PackedTensor:
         self.aux = torch.zeros(B, H, self.t_cap, (n * self.aux_bits + 7) // 8, **z) if self.aux_bits else None
         self.scale = torch.zeros(B, H, self.t_cap, dtype=dtype, device=self.device)
         self.joint = joint
+        # the largest finite scale written so far as fp32 bits (the quantize kernel keeps it up to date): the attention
+        # kernels' range guard for bf16 / fp32 caches; fp16 scales cannot leave the range
+        self.scale_max = None if dtype == torch.float16 else torch.zeros(1, dtype=torch.int32, device=self.device)
         self.length = 0                      # rows written when all sequences advance together
         self.lengths: Optional[torch.Tensor] = None  # per-sequence rows (int32, device) for ragged batches
         self.flags = self.sideband = self.sb_tile_off = self.sb_count = self.sb_overflow = self.sb_coord = None
@@ -87,6 +90,7 @@ class PackedTensor:
         s.sideband, s.sb_tile_off, s.sb_cap = L.ptr(self.sideband), L.ptr(self.sb_tile_off), self.sb_cap
         s.sb_coord, s.sb_count = L.ptr(self.sb_coord), L.ptr(self.sb_count)
         s.joint, s.joint_sh, s.K = L.ptr(self.joint), self.joint.stride(0), self.joint.shape[1]
+        s.scale_max_bits = L.ptr(self.scale_max)
         return s
 
     def crop_(self, lengths) -> None:

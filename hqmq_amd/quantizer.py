@@ -81,9 +81,17 @@ class HQMQQuantizer(KVQuantizer):
         self.training = training
         if tau is not None:
             self.tau = tau
+        self.invalidate_codebooks()
 
     def _refresh_rotations(self):
-        pass
+        self.invalidate_codebooks()
+
+    def invalidate_codebooks(self):
+        """Forget the cached joint tables.  They are rebuilt on the next call; needed after an in-place write
+        through secondary_raw.data (which leaves no trace on the parameter), not after assignments or ordinary
+        in-place ops, which the cache detects itself.  Packed caches made earlier keep the table they were created
+        with: codes stay decodable with the table they were encoded against."""
+        self._joint_cache.clear()
 
     # ---- codebook ----
     def _check_supported(self):
@@ -99,11 +107,12 @@ class HQMQQuantizer(KVQuantizer):
         if raw.device != ref.device:
             raise L.HqmqError(f"quantizer parameters are on {raw.device}, the tensor is on {ref.device}")
         key = (layer_idx, kv, ref.dtype)
+        stamp = (id(raw), raw.data_ptr(), raw._version)     # a new parameter, new storage (.data = w) or an in-place op
         hit = self._joint_cache.get(key)
-        if hit is not None and hit[0] == raw._version:
+        if hit is not None and hit[0] == stamp:
             return hit[1], hit[2]
         joint, slack = ops.build_joint(raw.detach()[layer_idx, :, kv], ref.dtype)
-        self._joint_cache[key] = (raw._version, joint, slack)
+        self._joint_cache[key] = (stamp, joint, slack)
         return joint, slack
 
     def _get_codebook(self, layer_idx: int, kv: int, ref: torch.Tensor) -> torch.Tensor:
@@ -248,6 +257,10 @@ class OutlierAwareHQMQQuantizer(KVQuantizer, _OutlierStats):
         assert isinstance(inner, HQMQQuantizer), "wrapper expects HQMQQuantizer"
         _OutlierStats.__init__(self)
         self.inner = inner
+        # The reference's median is torch.quantile, which raises above 2^24 chunks per head in one call
+        # (src/quantizers/outlier_aware.py:68).  The radix select here has no such bound; set this to True to get
+        # the reference's RuntimeError from quantize_K / quantize_V / encode instead of the extension.
+        self.strict_quantile_limit = False
         self.outlier_fraction, self.threshold_mode, self.median_mult = outlier_fraction, threshold_mode, median_mult
         self.chunk_dim = inner.chunk_dim
 
@@ -272,7 +285,7 @@ class OutlierAwareHQMQQuantizer(KVQuantizer, _OutlierStats):
             raise ValueError(f"d_head={x.shape[-1]} not divisible by 4")
         self.inner._check_supported()
         joint, slack = self.inner._joint_and_slack(layer_idx, kv, x)
-        _, thr, count = ops.med3x_threshold(x, self.median_mult)
+        _, thr, count = ops.med3x_threshold(x, self.median_mult, strict_quantile_limit=self.strict_quantile_limit)
         self._note(count, x.numel() // 4)
         return ops.quantize(x, joint, slack, self.inner.radius_bits, want_codes=False, want_dense=True, thr=thr)["out"]
 
@@ -303,7 +316,7 @@ class OutlierAwareHQMQQuantizer(KVQuantizer, _OutlierStats):
         self._require_median_mode()
         self.inner._check_supported()
         joint, slack = self.inner._joint_and_slack(layer_idx, kv, x)
-        med, thr, count = ops.med3x_threshold(x, self.median_mult)
+        med, thr, count = ops.med3x_threshold(x, self.median_mult, strict_quantile_limit=self.strict_quantile_limit)
         self._note(count, x.numel() // 4)
         out = ops.quantize(x, joint, slack, self.inner.radius_bits, want_codes=True, thr=thr, want_mask=True)
         out.update(joint=joint, median=med, threshold=thr)

@@ -97,6 +97,10 @@ typedef struct hqmq_quantize_args {
     const int32_t *pos;       /* [B] or NULL */
     int main_bits, aux_bits;
     int32_t *stats;           /* [2] or NULL, accumulated: lanes that scored all rows; secondaries kept by the filter */
+    uint32_t *scale_max_bits; /* [1] or NULL, accumulated (atomic max): the largest finite per-token scale written to
+                                 scale_plane, as the bits of an fp32 number; start it at 0.  The attention kernels read
+                                 it (hqmq_packed.scale_max_bits) to keep caches with scales beyond 2^15 inside the
+                                 fp16 range of their matrix products. */
 } hqmq_quantize_args;
 int hqmq_quantize(const hqmq_quantize_args *a, void *stream);
 
@@ -179,6 +183,11 @@ typedef struct hqmq_packed {
     const void *joint;        /* [H][K][4] D */
     int64_t joint_sh;         /* element stride between heads */
     int K;                    /* codewords in joint */
+    const uint32_t *scale_max_bits; /* [1] or NULL: an upper bound of the finite scales in scale_plane as fp32 bits, as
+                                 hqmq_quantize accumulates it.  Read for the V tensor of bf16 / fp32 caches: with a bound
+                                 above 2^15 the softmax weights are carried with a power-of-two offset, so that
+                                 P * scale stays finite in fp16 (the result is unchanged: numerator and denominator
+                                 carry the same factor).  NULL = all scales are below 2^15 (always true in fp16). */
 } hqmq_packed;
 
 /* Dense decode of a packed cache (outlier chunks substituted from the sideband).

@@ -247,3 +247,17 @@ def test_crop_bookkeeping_on_cpu():
     pt.crop_(20)                                                       # an int crops every sequence
     off3, cnt3 = state([20] * B)
     assert pt.length == 20 and np.array_equal(pt.sb_count.numpy(), cnt3) and np.array_equal(pt.sb_tile_off.numpy(), off3)
+
+
+def test_quantile_limit_check():
+    """The reference's Med-C median is torch.quantile, which refuses more than 2^24 elements per row
+    (src/quantizers/outlier_aware.py:68 of the reference); the check that mirrors it on request."""
+    from hqmq_amd import ops
+    assert ops.QUANTILE_LIMIT == 1 << 24
+    assert ops.check_quantile_limit(1 << 24, strict=True) is True
+    assert ops.check_quantile_limit((1 << 24) + 1, strict=False) is False
+    with pytest.raises(RuntimeError, match="too large"):
+        ops.check_quantile_limit((1 << 24) + 1, strict=True)
+    x = torch.zeros(2 ** 24 + 1)
+    with pytest.raises(RuntimeError, match="too large"):          # the behaviour being mirrored
+        torch.quantile(x, 0.5)
