@@ -110,7 +110,8 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
                            T_kv: Optional[int] = None, out: Optional[torch.Tensor] = None,
                            force_generic: bool = False, use_fp8_codebook: bool = False,
                            kv_starts: Optional[torch.Tensor] = None,
-                           batch_order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           batch_order: Optional[torch.Tensor] = None,
+                           fp8_table_storage: bool = False) -> torch.Tensor:
     """Fused attention straight from the bit-packed cache (the fast path).
 
     Decode: T_q = 1, causal=False.  Chunked prefill: causal=True with causal_offset = number of
@@ -119,8 +120,12 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
     e.g. ops.longest_first(kv_lens)) starts the sequences' blocks in that order: scheduling only, same result.
     force_generic runs the layout-generic kernel where a specialised one exists (a second implementation
     of the same arithmetic, used by the tests).  use_fp8_codebook decodes with the joint tables rounded to
-    float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache).
+    float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache);
+    with fp8_table_storage=True the kernel also keeps them as float8 in LDS (half the table footprint, two
+    conversions per gathered codeword; same results, slower on this GPU: see DESIGN.md).
     """
+    if fp8_table_storage and not use_fp8_codebook:
+        raise L.HqmqError("fp8_table_storage needs use_fp8_codebook=True: only tables rounded to e4m3 can be kept as float8")
     if use_fp8_codebook:
         cache = PackedKV(cache.K.with_fp8_table(), cache.V.with_fp8_table())
     if T_kv is None:
@@ -140,7 +145,7 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
         return O.contiguous()
     return ops.attn_fwd(Q, cache.K, cache.V, T_kv, kv_lens=kv_lens, kv_starts=kv_starts, batch_order=batch_order, causal=causal,
                         causal_offset=causal_offset, softmax_scale=softmax_scale, n_splits=n_splits, out=out,
-                        force_generic=force_generic)
+                        force_generic=force_generic, fp8_table_storage=fp8_table_storage)
 
 
 def fused_attention_reference(

@@ -48,6 +48,7 @@ struct AttnParams {
     int scale_vec;  // scales of 4 consecutive tokens may be read with one aligned vector load
     float *ws;      // split partials [row][split][kPartialHead + d_h]: m (base-2 exponent units), l, two unused floats, acc
     int xcd_remap;  // blocks of one (sequence, KV head) share an XCD (see attn_fast_kernel)
+    int tab_fp8;    // both tables hold e4m3 numbers and the caller asks for float8 storage in LDS
 };
 
 __device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {

@@ -40,9 +40,29 @@ __device__ __forceinline__ uint4v pair_to_half(uint4v w) {
     return uint4v{a.x, a.y, b.x, b.y};
 }
 
+// One codeword (four fp16 in two dwords) of e4m3 numbers -> four float8 bytes (exact)
+__device__ __forceinline__ uint32_t codeword_to_f8(uint32_t w0, uint32_t w1) {
+    const half2v a = __builtin_bit_cast(half2v, w0), b = __builtin_bit_cast(half2v, w1);
+    int v = __builtin_amdgcn_cvt_pk_fp8_f32((float)a[0], (float)a[1], 0, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32((float)b[0], (float)b[1], v, true);
+    return (uint32_t)v;
+}
+// Two codewords of a table whose entries are e4m3 numbers -> the same two as eight float8 bytes
+template <int DT>
+__device__ __forceinline__ uint2 pair_to_f8(uint4v w) {
+    const uint4v h = pair_to_half<DT>(w);
+    const uint32_t h0 = h[0], h1 = h[1], h2 = h[2], h3 = h[3];
+    return uint2{codeword_to_f8(h0, h1), codeword_to_f8(h2, h3)};
+}
+template <int DT, bool F8>
+__device__ __forceinline__ void store_pair(void *tab, int k, uint4v w) {
+    if constexpr (F8) reinterpret_cast<uint2 *>(tab)[k] = pair_to_f8<DT>(w);
+    else reinterpret_cast<uint4v *>(tab)[k] = pair_to_half<DT>(w);
+}
+
 // The rest of both per-head tables (pairs k0.. of K2 / V2 pairs) -> LDS as fp16, in batches of independent loads.
-template <int DT, int NT>
-__device__ __forceinline__ void fill_tables16(uint4v *kdst, const uint4v *ksrc, int Kk2, uint4v *vdst, const uint4v *vsrc, int Kv2, int k_first) {
+template <int DT, int NT, bool F8 = false>
+__device__ __forceinline__ void fill_tables16(void *kdst, const uint4v *ksrc, int Kk2, void *vdst, const uint4v *vsrc, int Kv2, int k_first) {
     constexpr int U = 3;
     for (int k0 = k_first + threadIdx.x; k0 < max(Kk2, Kv2); k0 += NT * U) {
         uint4v tk[U], tv[U];
@@ -55,8 +75,8 @@ __device__ __forceinline__ void fill_tables16(uint4v *kdst, const uint4v *ksrc, 
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = k0 + u * NT;
-            if (k < Kk2) kdst[k] = pair_to_half<DT>(tk[u]);
-            if (k < Kv2) vdst[k] = pair_to_half<DT>(tv[u]);
+            if (k < Kk2) store_pair<DT, F8>(kdst, k, tk[u]);
+            if (k < Kv2) store_pair<DT, F8>(vdst, k, tv[u]);
         }
     }
 }
@@ -168,13 +188,37 @@ __device__ __forceinline__ uint32_t half_addr8(uint32_t pair) {
     return r;
 }
 
+// The same for a table kept as float8 e4m3 (F8 variants: four bytes per codeword, for tables whose entries are e4m3
+// numbers): one 32-bit LDS read and two conversions that widen two bytes each to packed fp16 (exact).
+template <int TAB_OFF>
+__device__ __forceinline__ half4 gather4_f8(uint32_t byte_addr) {
+    const uint32_t w = *(lds_u1_ptr)(uintptr_t)(byte_addr + TAB_OFF);
+    const half2v lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    const half2v hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+    return half4{lo[0], lo[1], hi[0], hi[1]};
+}
+template <int HI>
+__device__ __forceinline__ uint32_t half_addr4(uint32_t pair) {
+    uint32_t r;
+    if constexpr (HI)
+        asm("v_lshlrev_b32_sdwa %0, 2, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1" : "=v"(r) : "v"(pair));
+    else
+        asm("v_lshlrev_b32_sdwa %0, 2, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0" : "=v"(r) : "v"(pair));
+    return r;
+}
+template <int TAB_OFF, bool F8, int HI>
+__device__ __forceinline__ half4 gather_pair_half(uint32_t ix) {
+    if constexpr (F8) return gather4_f8<TAB_OFF>(half_addr4<HI>(ix));
+    else return gather8<TAB_OFF>(half_addr8<HI>(ix));
+}
+
 // Decode of the CPL chunks of one lane in two steps, so that a caller can put all gathers of a half-step in flight
 // before the first multiply: gather_chunks requests the codewords from the LDS table (g) and prepares the radius
 // codes as packed fp16 pairs (r, chunk j in r[j / 2][j & 1]); scale_chunks multiplies.
 // 16+0 layout: the two radius codes of a dword become an fp16 pair with one shift, one and-or
 // (0x6400 | rq is the fp16 number 1024 + rq) and one packed subtract.  IB = idx_bits when known at compile
 // time (12 for s96), else 0.
-template <int CPL, int MB, int AB, int IB, int NW, int TAB_OFF>
+template <int CPL, int MB, int AB, int IB, int NW, int TAB_OFF, bool F8 = false>
 __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t aux, int idx_bits_rt, half4 (&g)[CPL], half2v (&r)[CPL / 2]) {
     const int idx_bits = IB ? IB : idx_bits_rt;
     const uint32_t idx_mask = (1u << idx_bits) - 1u;
@@ -188,8 +232,8 @@ __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t 
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
-            g[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix));
-            g[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix));
+            g[2 * i] = gather_pair_half<TAB_OFF, F8, 0>(ix);
+            g[2 * i + 1] = gather_pair_half<TAB_OFF, F8, 1>(ix);
             const uint32_t t = ((w[i] >> idx_bits) & rq2) | magic;
             r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
@@ -201,13 +245,14 @@ __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t 
 #pragma unroll
         for (int i = 0; i < CPL / 2; i++) {
             const uint32_t ix = w[i] & im2;
-            g[2 * i] = gather8<TAB_OFF>(half_addr8<0>(ix));
-            g[2 * i + 1] = gather8<TAB_OFF>(half_addr8<1>(ix));
+            g[2 * i] = gather_pair_half<TAB_OFF, F8, 0>(ix);
+            g[2 * i + 1] = gather_pair_half<TAB_OFF, F8, 1>(ix);
             const uint32_t hi = *(lds_u1_ptr)(uintptr_t)(kAuxTabOffset + ((aux >> (6 * i)) & 63u) * 4u);
             const uint32_t t = ((w[i] >> 13) & 0x00070007u) | hi;
             r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
     } else if constexpr (MB == 12 && AB == 1 && IB == 10 && CPL == 8) {
+        static_assert(!F8, "the float8 table variants exist for 16-bit main fields");
         // s24_r3: eight 12-bit fields (idx in the low 10 bits, the low two radius bits above) in three dwords
         // and one aux byte with the eight high radius bits.  The aux byte indexes a 256-entry LDS table whose row
         // holds, per pair of chunks, the two high radius bits at bits 2 and 18 and the 0x6400 fp16 magic.
@@ -228,6 +273,7 @@ __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t 
             r[i] = __builtin_bit_cast(half2v, t) - k1024;
         }
     } else {
+        static_assert(!F8, "the float8 table variants exist for the layouts with compile-time index widths");
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             uint32_t code = code_at<MB, NW>(w, j);
@@ -272,7 +318,8 @@ __device__ __forceinline__ half4 pack4(float4v t) {
 
 // NCG: column groups (of 16 columns) per wavefront.  Two for chunked prefill with more than 16 columns per KV head:
 // a decoded tile and its V transposition then serve 32 columns.
-template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS, int WV = kFastWaves, int NCG = 1>
+// F8: the codeword tables are kept as float8 e4m3 in LDS (callers that rounded their tables to e4m3)
+template <int CPL, int MB, int AB, int IB, int DT, bool FLAGS, int WV = kFastWaves, int NCG = 1, bool F8 = false>
 __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(AttnParams p) {
     static_assert(NCG == 1 || !FLAGS, "outlier variants take one column group");
     constexpr int NB = CPL * MB / 8;
@@ -462,14 +509,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     for (int e = 0; e < 4; e++) ident_bf[e] = (short)((4 * grp + e) == col ? 0x3F80 : 0);
 
     {
-        uint4v *ktab4 = reinterpret_cast<uint4v *>(ktab), *vtab4 = reinterpret_cast<uint4v *>(vtab);
 #pragma unroll
         for (int u = 0; u < FU; u++) {
             const int k = threadIdx.x + u * NT;
-            if (k < Kk2) ktab4[k] = pair_to_half<DT>(tk[u]);
-            if (k < Kv2) vtab4[k] = pair_to_half<DT>(tv[u]);
+            if (k < Kk2) store_pair<DT, F8>(ktab, k, tk[u]);
+            if (k < Kv2) store_pair<DT, F8>(vtab, k, tv[u]);
         }
-        if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT>(ktab4, ksrc, Kk2, vtab4, vsrc, Kv2, FU * NT);
+        if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT, F8>(ktab, ksrc, Kk2, vtab, vsrc, Kv2, FU * NT);
     }
     // Plain variants keep two half-steps in flight.  The second one is requested only now, when the table loads
     // have come back: requested at the start it would queue in front of them and delay the whole block.
@@ -671,13 +717,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         half2v rk[2][CPL / 2];
         if constexpr (kBatchGathers) {
 #pragma unroll
-            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
+            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, 0, F8>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
-            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, 0>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
+            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, 0, F8>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
             scale_chunks<CPL>(gk[u], rk[u], a);
 #pragma unroll
             for (int cgi = 0; cgi < NCG; cgi++) {
@@ -696,7 +742,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         half2v rv[2][CPL / 2];
         if constexpr (kBatchGathers) {
 #pragma unroll
-            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
         // ---- mask (boundary half-steps only), online softmax, per column group ----
@@ -758,7 +804,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         half4 av[2][CPL];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
             scale_chunks<CPL>(gv[u], rv[u], av[u]);
         }
 #pragma unroll
@@ -875,7 +921,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     }
 }
 
-template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves, int NCG = 1>
+template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves, int NCG = 1, bool F8 = false>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
     if (NCG > 1) grid.y = (grid.y + NCG - 1) / NCG;
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
@@ -883,7 +929,7 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st
     const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);     // WV >= the wavefronts actually launched
     if (shmem < merge) shmem = merge;
     constexpr int WF = CPL == 4 ? WV : kFastWaves;      // outlier variants fit three wavefronts per SIMD only at d_h 64
-    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, WF> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV, NCG>;
+    auto kern = flags ? attn_fast_kernel<CPL, MB, AB, IB, DT, true, WF, 1, F8> : attn_fast_kernel<CPL, MB, AB, IB, DT, false, WV, NCG, F8>;
     if (shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
@@ -907,6 +953,11 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     // chunked prefill (more than 16 columns per KV head) of plain caches: two column groups per wavefront
     // (only while a block per CU is left: fewer, larger blocks lose more than the shared decode wins)
     const bool two = !flags && p.n_cg > 1 && (int64_t)p.n_splits * ((p.n_cg + 1) / 2) * p.B * p.Hkv >= 256;
+    // tables of e4m3 numbers kept as float8 in LDS, on request (decode shapes of the 16-bit layouts at d_h 128)
+    if (p.tab_fp8 && CPL == 8 && !two) {
+        if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<8, 16, 0, 12, DT, kFastWaves, 1, true>(p, flags, grid, st, tm);
+        if (mb == 16 && p.aux_bits == 3 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT, kFastWaves, 1, true>(p, flags, grid, st, tm);
+    }
     if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) {
         if (two) return launch_one<CPL, 16, 0, 12, DT, kFastWaves, 2>(p, flags, grid, st, tm);
         return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);

@@ -309,12 +309,14 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
              causal_offset: int = 0, softmax_scale: Optional[float] = None, n_splits: int = 0,
              out: Optional[torch.Tensor] = None, skip_combine: bool = False,
              force_generic: bool = False, kernel_events: Optional[tuple] = None,
-             static_scratch: bool = False, workspace: Optional[torch.Tensor] = None):
+             static_scratch: bool = False, workspace: Optional[torch.Tensor] = None, fp8_table_storage: bool = False):
     """Fused attention of Q (B, H_q, T_q, d_h) over packed K/V (PackedTensor each).
     kernel_events: two raw hipEvent_t handles (ints) that receive the GPU timestamps of the begin and the end of
     the main attention kernel (profiling).
     static_scratch: call hqmq_attn_fwd_static, which keeps the split partials in the library's own device array
     instead of a torch workspace (pass `out` as well and the call allocates nothing on the device).
+    fp8_table_storage: both joint tables hold float8 e4m3 numbers (PackedTensor.with_fp8_table) and the kernel may keep
+    them as float8 in LDS; same results, see include/hqmq_amd.h.
     skip_combine: leave the split partials unmerged and return (O, partials, n_splits): the partials are in `workspace`
     if given, else in a buffer of their own (never the cached scratch that the next call on the stream overwrites);
     attn_combine(partials, O, n_splits) merges them."""
@@ -363,6 +365,7 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     a.n_splits = n_splits
     a.skip_combine = int(skip_combine)
     a.force_generic = int(force_generic)
+    a.fp8_table_storage = int(fp8_table_storage)
     if kernel_events is not None:
         a.start_event, a.stop_event = C.c_void_p(kernel_events[0]), C.c_void_p(kernel_events[1])
     ws = None

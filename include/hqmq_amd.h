@@ -225,6 +225,11 @@ typedef struct hqmq_attn_args {
                                    started (pass the sequences sorted by length, longest first, for ragged batches) */
     void *start_event, *stop_event; /* hipEvent_t or NULL: receive the GPU timestamps of the begin and the end of
                                        the main attention kernel (hipEventElapsedTime = its duration; profiling) */
+    int fp8_table_storage;    /* 1: every entry of both joint tables is a float8 e4m3 number (the caller rounded them, as
+                                 the reference's use_fp8_codebook does, src/quantizers/hqmq_attention_hopper.py:43-53) and
+                                 the kernel may keep them as float8 in LDS (4 bytes per codeword, widened after the
+                                 gather as :133-135 there does).  Same results as 0 on such tables; honoured by the
+                                 specialised decode kernels of the 16-bit layouts at d_h 128, ignored elsewhere. */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
 /* The n_splits hqmq_attn_fwd would choose; ragged = 1 when kv_len is passed (more, smaller blocks). */

@@ -133,3 +133,31 @@ def test_padded_quantizer_packed_path(d_head, S, b_r):
     s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_head ** -0.5
     ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
     assert O.shape == Q.shape and (O.float() - ref).abs().max().item() < 2e-3
+
+
+@pytest.mark.parametrize("S,b_r,dn,outl", [(96, 4, "fp16", False), (192, 6, "fp16", True), (192, 6, "bf16", False), (96, 4, "bf16", True)])
+def test_fp8_table_storage_gives_the_same_result(S, b_r, dn, outl):
+    """use_fp8_codebook rounds the joint tables to e4m3; fp8_table_storage additionally keeps them as float8 in LDS
+    (the reference's Hopper path stores fp8 and promotes after the gather, hqmq_attention_hopper.py:43-53,133-135).
+    Every e4m3 number is exact in fp16, so the two storages must agree bit for bit."""
+    import hqmq
+    dt = torch.float16 if dn == "fp16" else torch.bfloat16
+    B, Hq, Hkv, T, d_h = 2, 8, 2, 1500, 128
+    g = torch.Generator().manual_seed(S)
+    k, v = torch.randn(B, Hkv, T, d_h, generator=g), torch.randn(B, Hkv, T, d_h, generator=g)
+    if outl:
+        k[:, :, ::7, 8:12] *= 30.0
+        v[:, :, ::5, 64:68] *= 20.0
+    q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV)
+    w = hqmq.with_outlier_extraction(q, C=3.0) if outl else q
+    cache = w.new_cache(B, T, d_h, dt, 0, **({"sideband_frac": 0.25} if outl else {}))
+    w.append(cache, k.to(dt).to(DEV), v.to(dt).to(DEV), 0)
+    Q = torch.randn(B, Hq, 1, d_h, generator=g).to(dt).to(DEV)
+    plain = hqmq.fused_attention_packed(Q, cache)
+    for ns in (0, 1, 3):
+        a = hqmq.fused_attention_packed(Q, cache, use_fp8_codebook=True, n_splits=ns)
+        b = hqmq.fused_attention_packed(Q, cache, use_fp8_codebook=True, fp8_table_storage=True, n_splits=ns)
+        assert torch.equal(a, b), ns
+        assert not torch.equal(a, plain)
+    with pytest.raises(hqmq.HqmqError):
+        hqmq.fused_attention_packed(Q, cache, fp8_table_storage=True)
