@@ -342,12 +342,12 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const flo
 #pragma unroll
             for (int i = 0; i < SC; i++) mx = fmaxf(mx, ml[i].x);
             if (mx > -INFINITY) {
-                const float f = exp2f(M - mx);          // 0 while M is still -inf
+                const float f = __builtin_amdgcn_exp2f(M - mx);          // 0 while M is still -inf
                 L *= f;
                 A = A * f;
 #pragma unroll
                 for (int i = 0; i < SC; i++) {
-                    const float w = exp2f(ml[i].x - mx);
+                    const float w = __builtin_amdgcn_exp2f(ml[i].x - mx);
                     L = fmaf(ml[i].y, w, L);
                     A = A + as[i] * w;
                 }
@@ -359,15 +359,24 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const flo
     }
     __syncthreads();
     if (grp != 0) return;
-    for (int g = 1; g < groups; g++) {
-        const float *r = red + (size_t)(g * ncol + c4) * 6;
-        const float m2 = r[0];
-        const float mx = fmaxf(M, m2);
-        if (mx > -INFINITY) {
-            const float f = exp2f(M - mx), w = exp2f(m2 - mx);
-            L = fmaf(r[1], w, L * f);
-            A = A * f + float4v{r[2], r[3], r[4], r[5]} * w;
-            M = mx;
+    // the groups' results: the maximum first (independent reads), then one weight per group, in batches of eight
+    float mx = M;
+    for (int g = 1; g < groups; g++) mx = fmaxf(mx, red[(size_t)(g * ncol + c4) * 6]);
+    if (mx > -INFINITY) {
+        const float f = __builtin_amdgcn_exp2f(M - mx);
+        L *= f;
+        A = A * f;
+        for (int g0 = 1; g0 < groups; g0 += 8) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int g = g0 + i;
+                if (g < groups) {
+                    const float *r = red + (size_t)(g * ncol + c4) * 6;
+                    const float w = __builtin_amdgcn_exp2f(r[0] - mx);      // -inf - finite = -inf -> 0
+                    L = fmaf(r[1], w, L);
+                    A = A + float4v{r[2], r[3], r[4], r[5]} * w;
+                }
+            }
         }
     }
     const unsigned bh = row / (unsigned)Tq, tq = row - bh * (unsigned)Tq, b = bh / (unsigned)Hq, hq = bh - b * (unsigned)Hq;

@@ -232,11 +232,15 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 a_next = acol[4 * min(s + slots, S - 1)];       // the next column is on its way during this one
                 const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 const float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
-                asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
-                if (b2 >= m2 - margin2) {
+                // kept: within the margin of the running maximum.  A score that beats the old maximum by more than the
+                // margin leaves everything kept so far more than the margin below the final maximum: the list starts
+                // over, which keeps it at the true candidates instead of every record of the scan.
+                if (b2 + margin2 >= m2) {
+                    if (b2 - margin2 > m2) cnt = 0;
                     if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
                     cnt++;
                 }
+                asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
             }
         } else {
             for (int s = 0; s < S; s++) {
@@ -244,11 +248,12 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 float v[4];
                 rotate_conj(us, q.x, q.y, q.z, q.w, v);
                 const float b2 = best2_of(v);
-                m2 = fmaxf(m2, b2);
-                if (b2 >= m2 - margin2) {
+                if (b2 + margin2 >= m2) {
+                    if (b2 - margin2 > m2) cnt = 0;
                     if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
                     cnt++;
                 }
+                m2 = fmaxf(m2, b2);
             }
         }
         if (SPLIT) {        // the maximum over all slots of this chunk (every slot holds the same direction)
