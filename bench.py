@@ -274,6 +274,12 @@ def main():
     us_launch_interval, _ = graph_us(lambda i: main_kernel(i, None), args.steps, stream)
     us_step_same, _ = graph_us(step_same, args.steps, stream)
     achieved = cache_bytes / (us_main * 1e-6) / 1e9
+    # what the memory system allows a launch of this shape: the kernel that only reads the same planes with the same
+    # grid, per-wavefront ranges and loads (hqmq_attn_read_ceiling), caches rotating / one cache
+    us_read = kernel_time_us(lambda i, ev: ops.read_ceiling(caches[i % NL].K, caches[i % NL].V, T, H_q=Hq, n_splits=n_splits,
+                                                             depth=3, waves=8, kernel_events=ev), 192)
+    us_read_same = kernel_time_us(lambda i, ev: ops.read_ceiling(caches[0].K, caches[0].V, T, H_q=Hq, n_splits=n_splits,
+                                                                  depth=3, waves=8, kernel_events=ev), 192)
 
     result = {
         "metric": "decode-attn HBM GB/s on compressed bytes (us/step and % of 8 TB/s alongside); quantize GTok/s",
@@ -303,12 +309,16 @@ def main():
                                        f"measured by this run)" if T in RECORDED_TRAFFIC_BYTES else None,
                      "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1>", "kernel_us": round(us_main, 2),
                      "kernel_launch_interval_us": round(us_launch_interval, 2),
-                     "algorithmic_bytes_per_launch": cache_bytes},
+                     "algorithmic_bytes_per_launch": cache_bytes,
+                     "read_only_kernel_same_grid_us": round(us_read, 2),
+                     "read_only_kernel_GBps": round(cache_bytes / us_read / 1e3, 1),
+                     "frac_of_read_only_kernel": round(us_read / us_main, 4)},
         "same_cache_replay": {
             "what": "the same step over ONE cache replayed back to back: its 34.6 MB stay in the L2s and the 256 MB "
                     "Infinity Cache, so this is not an HBM figure; reported as the cache-resident upper bound",
             "us_per_step": round(us_step_same, 2), "GBps": round(step_bytes / us_step_same / 1e3, 1),
-            "kernel_us": round(us_main_same, 2), "kernel_GBps": round(cache_bytes / us_main_same / 1e3, 1)},
+            "kernel_us": round(us_main_same, 2), "kernel_GBps": round(cache_bytes / us_main_same / 1e3, 1),
+            "read_only_kernel_same_grid_us": round(us_read_same, 2)},
     }
     if not args.quick:
         # quantize throughput: K and V of one layer, bulk (prefill) call, packed output

@@ -67,7 +67,7 @@ class AttnArgs(C.Structure):
         ("kv_len", vp), ("causal", C.c_int), ("causal_offset", i64), ("softmax_scale", C.c_float),
         ("n_splits", C.c_int), ("workspace", vp), ("workspace_bytes", i64), ("skip_combine", C.c_int), ("force_generic", C.c_int),
         ("kv_start", vp), ("batch_order", vp), ("start_event", vp), ("stop_event", vp),
-        ("fp8_table_storage", C.c_int),
+        ("fp8_table_storage", C.c_int), ("wide_range", C.c_int),
     ]
 
 

@@ -54,6 +54,8 @@ def _pack_unpacked(idx, rq, rs, joint, r_qmax: int) -> PackedTensor:
     pt.scale[:, :, :T] = rs            # into the padded plane: rows up to the capacity stay readable
     if pt.scale_max is not None:       # the range guard of bf16 / fp32 caches: the largest finite scale, as fp32 bits
         pt.scale_max = torch.nan_to_num(rs.detach().float().abs(), nan=0.0, posinf=0.0).amax().reshape(1).view(torch.int32)
+        if pt.dtype == torch.bfloat16 and not torch.cuda.is_current_stream_capturing():
+            pt.refresh_range()         # one device read: bf16 scales of 2^15 and more take the guarded kernel
     pt.length = T
     return pt
 

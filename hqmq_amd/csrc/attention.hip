@@ -522,6 +522,7 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     // Ragged batches keep the sequence-major order that batch_order relies on.
     p.xcd_remap = (!a->kv_len && !a->batch_order && ((a->B * a->H_kv) % 8) == 0) ? 1 : 0;
     p.tab_fp8 = a->fp8_table_storage ? 1 : 0;
+    p.wide_range = a->wide_range ? 1 : 0;
     // 4 consecutive scales with one vector load: unit stride, aligned rows, and capacity rows readable
     const int salign = a->dtype == HQMQ_F32 ? 16 : 8;
     p.scale_vec = 1;

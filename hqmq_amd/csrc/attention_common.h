@@ -49,6 +49,7 @@ struct AttnParams {
     float *ws;      // split partials [row][split][kPartialHead + d_h]: m (base-2 exponent units), l, two unused floats, acc
     int xcd_remap;  // blocks of one (sequence, KV head) share an XCD (see attn_fast_kernel)
     int tab_fp8;    // both tables hold e4m3 numbers and the caller asks for float8 storage in LDS
+    int wide_range; // scales or verbatim values of the cache may leave the fp16 range: layout-generic kernel only
 };
 
 __device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {
@@ -201,12 +202,13 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
 
 // Power-of-two offset of the softmax exponent that keeps P * (V scale) inside fp16: 0 while the largest V scale is
 // below 2^15, else its excess exponent.  Numerator and denominator of the attention output carry the same factor.
-__device__ __forceinline__ float v_scale_shift(const PackedDev &v) {
-    if (!v.scale_max) return 0.f;
-    const uint32_t bits = __builtin_nontemporal_load(v.scale_max);
+__device__ __forceinline__ int v_scale_shift_bits(const PackedDev &v) {
+    if (!v.scale_max) return 0;
+    const uint32_t bits = __builtin_amdgcn_readfirstlane(__builtin_nontemporal_load(v.scale_max));      // wave-uniform
     const int e = (int)((bits >> 23) & 0xffu) - 127 + 1;        // scale < 2^e
-    return (float)max(e - 15, 0);
+    return max(e - 15, 0);
 }
+__device__ __forceinline__ float v_scale_shift(const PackedDev &v) { return (float)v_scale_shift_bits(v); }
 
 // Implemented in attention_fast.hip: kernels specialised at compile time for the common layouts
 // (d_h 64/128, fp16/bf16 caches, 16+0 / 12+1 / 16+3 bit codes). Returns HQMQ_OK and sets *handled when

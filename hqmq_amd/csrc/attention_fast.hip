@@ -567,7 +567,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 
     // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
     const float c = p.c_log2, qmaxf = (float)p.qmax;
-    const float eshift = DT == HQMQ_F16 ? 0.f : v_scale_shift(p.Vc);       // see attention_common.h
     float m_run[NCG], l_run[NCG];
     float4v acc[NCG][CPL];
 #pragma unroll
@@ -662,8 +661,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const uint32_t slot = (e >= off[1] ? 4u : 0u) + (t & 3u);             // position among the row group's 8 tokens
         const bool mine = ok && (int)(t >> 2) == grp;
         const uint4v sel = *(lds_u4_ptr)(uintptr_t)(kSelOffset + (mine ? slot : 8u) * 16u);
-        const float4v pgf = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0);
-        const half4 pg = pack4(pgf);
+        const half4 pg = pack4(__builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0));
         half4 h = zero_h4;
         if constexpr (!kBfEntries) h = chunk_to_half<DT>(x);
         const bool owner = ok && (int)(ch / CPL) == grp;
@@ -677,18 +675,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                     tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, mj ? x : uint2{0u, 0u}), ident_bf, zero4, 0, 0, 0);
                 else
                     tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
-                if (kBfEntries && eshift != 0.f) {
-                    // a cache whose values leave the fp16 range (wave-uniform, never taken otherwise): the verbatim
-                    // chunks stay bf16 (tr holds them exactly) and the weights are rounded to bf16 for this product
-                    const uint32_t t01 = __builtin_amdgcn_perm(__float_as_uint(tr[1]), __float_as_uint(tr[0]), 0x07060302u);
-                    const uint32_t t23 = __builtin_amdgcn_perm(__float_as_uint(tr[3]), __float_as_uint(tr[2]), 0x07060302u);
-                    const uint32_t g01 = (uint32_t)f32_to_bf16_bits(pgf[0]) | (uint32_t)f32_to_bf16_bits(pgf[1]) << 16;
-                    const uint32_t g23 = (uint32_t)f32_to_bf16_bits(pgf[2]) | (uint32_t)f32_to_bf16_bits(pgf[3]) << 16;
-                    acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, uint2{t01, t23}),
-                                                                          __builtin_bit_cast(short4v, uint2{g01, g23}), acc[0][j], 0, 0, 0);
-                } else {
-                    acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
-                }
+                acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
             }
         }
     };
@@ -772,7 +759,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 for (int j = 0; j < CPL; j++) acc[cgi][j] = acc[cgi][j] * alpha;
                 m_run[cgi] = m_new;
             }
-            const float mc = -m_use * c - eshift;
+            const float mc = -m_use * c;
             half4 pT[2];
 #pragma unroll
             for (int u = 0; u < 2; u++) {
@@ -782,20 +769,11 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                     pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[cgi][u][e], c, mc));
                     l_run[cgi] += pe[e];
                 }
-                if constexpr (DT == HQMQ_F16) {
-                    const half2v u01 = half2v{(_Float16)pe[0], (_Float16)pe[1]}, u23 = half2v{(_Float16)pe[2], (_Float16)pe[3]};
-                    const half2v p01 = u01 * scale_h2<DT>(h.vs[u].x);
-                    const half2v p23 = u23 * scale_h2<DT>(h.vs[u].y);
-                    pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
-                    if (FLAGS) pTo[u] = half4{u01[0], u01[1], u23[0], u23[1]};      // unscaled: the selector rows hold qmax
-                } else {
-                    // bf16 scales reach beyond the fp16 range: the product is formed in fp32 (the exponent offset of the
-                    // softmax weights keeps it below 2^15) and only then rounded to fp16; same number of operations
-                    const uint32_t s01 = h.vs[u].x, s23 = h.vs[u].y;
-                    pT[u] = half4{(_Float16)(pe[0] * __uint_as_float(s01 << 16)), (_Float16)(pe[1] * __uint_as_float(s01 & 0xffff0000u)),
-                                  (_Float16)(pe[2] * __uint_as_float(s23 << 16)), (_Float16)(pe[3] * __uint_as_float(s23 & 0xffff0000u))};
-                    if (FLAGS) pTo[u] = half4{(_Float16)pe[0], (_Float16)pe[1], (_Float16)pe[2], (_Float16)pe[3]};
-                }
+                const half2v u01 = half2v{(_Float16)pe[0], (_Float16)pe[1]}, u23 = half2v{(_Float16)pe[2], (_Float16)pe[3]};
+                const half2v p01 = u01 * scale_h2<DT>(h.vs[u].x);
+                const half2v p23 = u23 * scale_h2<DT>(h.vs[u].y);
+                pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
+                if (FLAGS) pTo[u] = half4{u01[0], u01[1], u23[0], u23[1]};      // unscaled: the selector rows hold qmax
             }
             pp[cgi] = cat8(pT[0], pT[1]);
         }
@@ -984,6 +962,9 @@ int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, 
     (void)table_bytes;
     *handled = false;
     if (p.dtype != HQMQ_F16 && p.dtype != HQMQ_BF16) return HQMQ_OK;
+    // The kernels of this file form P * (V scale) and convert verbatim chunks in fp16: a bf16 cache whose scales reach
+    // 2^15 (the caller says so: wide_range) takes the layout-generic kernel, which carries the range guard.
+    if (p.wide_range) return HQMQ_OK;
     if (p.n != 16 && p.n != 32) return HQMQ_OK;
     if (p.t_cap % kSuper) return HQMQ_OK;
     // vector loads of plane rows: main rows 16-byte aligned (checked by the caller), aux and flag rows to their width

@@ -47,6 +47,11 @@ class PackedTensor:
         # the largest finite scale written so far as fp32 bits (the quantize kernel keeps it up to date): the attention
         # kernels' range guard for bf16 / fp32 caches; fp16 scales cannot leave the range
         self.scale_max = None if dtype == torch.float16 else torch.zeros(1, dtype=torch.int32, device=self.device)
+        # host-side copy of "scale_max has reached 2^15": such a cache takes the layout-generic attention kernel, which
+        # guards the fp16 range (refresh_range reads the device value; the quantizer calls it after bulk appends and
+        # every RANGE_CHECK_EVERY small ones)
+        self.wide_range = False
+        self._appends_since_range_check = 0
         self.length = 0                      # rows written when all sequences advance together
         self.lengths: Optional[torch.Tensor] = None  # per-sequence rows (int32, device) for ragged batches
         self.flags = self.sideband = self.sb_tile_off = self.sb_count = self.sb_overflow = self.sb_coord = None
@@ -92,6 +97,25 @@ class PackedTensor:
         s.joint, s.joint_sh, s.K = L.ptr(self.joint), self.joint.stride(0), self.joint.shape[1]
         s.scale_max_bits = L.ptr(self.scale_max)
         return s
+
+    RANGE_CHECK_EVERY = 256
+
+    def refresh_range(self) -> bool:
+        """Reads the largest scale written so far (one device read) and records whether it has reached 2^15, the
+        bound above which the specialised attention kernels would leave the fp16 range.  Only ever switches on."""
+        if self.scale_max is not None and not self.wide_range:
+            self.wide_range = float(self.scale_max.view(torch.float32).item()) >= 32768.0
+        self._appends_since_range_check = 0
+        return self.wide_range
+
+    def note_append(self, rows: int) -> None:
+        """Called by the quantizer after an append of `rows` rows per sequence: bulk appends (a prefill) and every
+        RANGE_CHECK_EVERY-th small one refresh the range flag; never while the stream is being captured."""
+        if self.scale_max is None or self.wide_range:
+            return
+        self._appends_since_range_check += 1
+        if (rows >= 64 or self._appends_since_range_check >= self.RANGE_CHECK_EVERY) and not torch.cuda.is_current_stream_capturing():
+            self.refresh_range()
 
     def crop_(self, lengths) -> None:
         """Forgets the rows from `lengths` on (an int for all sequences or an int tensor [B]): the outlier list and

@@ -196,6 +196,7 @@ class HQMQQuantizer(KVQuantizer):
             ops.outlier_compact(x, cache, t_off=t_off, pos=pos)
         if pos is None:
             cache.length = t_off + T
+        cache.note_append(T)
         return count
 
     def append(self, cache: PackedKV, k: torch.Tensor, v: torch.Tensor, layer_idx: int,
@@ -225,6 +226,8 @@ class HQMQQuantizer(KVQuantizer):
                                median_mult=median_mult)
         if pos is None:
             cache.K.length = cache.V.length = t_off + T
+        cache.K.note_append(T)
+        cache.V.note_append(T)
         return counts
 
 

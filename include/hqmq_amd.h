@@ -184,10 +184,11 @@ typedef struct hqmq_packed {
     int64_t joint_sh;         /* element stride between heads */
     int K;                    /* codewords in joint */
     const uint32_t *scale_max_bits; /* [1] or NULL: an upper bound of the finite scales in scale_plane as fp32 bits, as
-                                 hqmq_quantize accumulates it.  Read for the V tensor of bf16 / fp32 caches: with a bound
-                                 above 2^15 the softmax weights are carried with a power-of-two offset, so that
-                                 P * scale stays finite in fp16 (the result is unchanged: numerator and denominator
-                                 carry the same factor).  NULL = all scales are below 2^15 (always true in fp16). */
+                                 hqmq_quantize accumulates it.  Read by the layout-generic attention kernel (see
+                                 hqmq_attn_args.wide_range): with a bound of 2^15 or more the softmax weights are carried
+                                 with a power-of-two offset and verbatim outlier chunks are rescaled, so that every
+                                 product stays finite in fp16 (the result is unchanged: numerator and denominator carry
+                                 the same factor).  NULL = all scales are below 2^15 (always true in fp16). */
 } hqmq_packed;
 
 /* Dense decode of a packed cache (outlier chunks substituted from the sideband).
@@ -230,6 +231,12 @@ typedef struct hqmq_attn_args {
                                  the kernel may keep them as float8 in LDS (4 bytes per codeword, widened after the
                                  gather as :133-135 there does).  Same results as 0 on such tables; honoured by the
                                  specialised decode kernels of the 16-bit layouts at d_h 128, ignored elsewhere. */
+    int wide_range;           /* 1: a bf16 cache whose per-token scales may reach 2^15 (or whose verbatim outlier values may
+                                 exceed 65504).  The specialised kernels multiply the softmax weights with the V scales in
+                                 fp16 and would overflow; such a cache takes the layout-generic kernel, which reads
+                                 hqmq_packed.scale_max_bits and keeps every product inside the fp16 range (fp32 caches always
+                                 take it).  Callers that track the bound (hqmq_quantize_args.scale_max_bits) set this when it
+                                 reaches 2^15; data of ordinary magnitude never does. */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
 /* The n_splits hqmq_attn_fwd would choose; ragged = 1 when kv_len is passed (more, smaller blocks). */

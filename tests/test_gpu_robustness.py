@@ -13,10 +13,11 @@ DEV = "cuda"
 @pytest.mark.parametrize("k_gain,v_gain", [(1.0, 1e5), (1e5, 1e5), (1e-3, 3e7)])
 @pytest.mark.parametrize("med3x", [False, True])
 def test_bf16_scales_beyond_fp16_range(k_gain, v_gain, med3x):
-    """bf16 K / V far outside the fp16 range (per-token scales up to ~1e9): the kernels carry the K scale in fp32 and
-    the softmax weights with a power-of-two offset taken from the cache's largest V scale, so P * scale stays finite
-    in the fp16 matrix products.  Checked against the CPU oracle, specialised and layout-generic kernels, packed and
-    unpacked entry points."""
+    """bf16 K / V far outside the fp16 range (per-token scales up to ~1e9).  The quantize kernel tracks the largest
+    scale; once it reaches 2^15 the cache is marked wide_range and attention takes the layout-generic kernel, which
+    carries the K scale in fp32, the softmax weights with a power-of-two offset taken from that bound and the verbatim
+    chunks rescaled, so every fp16 matrix product stays finite.  Checked against the CPU oracle through the packed
+    and the unpacked entry points."""
     import hqmq
     from hqmq_amd import ops
     dt = torch.bfloat16
@@ -31,6 +32,7 @@ def test_bf16_scales_beyond_fp16_range(k_gain, v_gain, med3x):
     assert float(cache.V.scale.float().max()) > 65504.0                      # beyond fp16
     vmax = cache.V.scale_max.view(torch.float32)
     assert float(vmax) == float(cache.V.scale[:, :, :T].float().max())       # the quantize kernel tracked the maximum
+    assert cache.V.wide_range                                                # read back after the bulk append
     qmax = (1 << b_r) - 1
     dense = {}
     for tag, x, kv in (("K", k, 0), ("V", v, 1)):
@@ -157,3 +159,25 @@ def test_strict_quantile_limit_mirrors_the_reference(monkeypatch):
     with pytest.raises(RuntimeError, match="quantile\\(\\) input tensor is too large"):
         w.quantize_K(x, 0)
     w.quantize_K(x[:, :, :30], 0)                                  # 960 chunks per head: within the limit
+
+
+def test_range_flag_follows_decode_appends():
+    """A cache of ordinary magnitude stays on the specialised kernels; a later token with a huge scale is noticed at
+    the next range check (every RANGE_CHECK_EVERY small appends, or on request) and moves it to the guarded kernel."""
+    import hqmq
+    dt = torch.bfloat16
+    q = hqmq.HQMQ(n_layers=1, n_heads=2, secondary_size=96, radius_bits=4, device=DEV)
+    cache = q.new_cache(1, 512, 128, dt, 0)
+    x = kv_input((1, 2, 300, 128), dt, 5).to(DEV)
+    q.append(cache, x, x, 0)
+    assert not cache.V.wide_range
+    Q = torch.randn(1, 8, 1, 128, generator=torch.Generator().manual_seed(6)).to(dt).to(DEV)
+    base = hqmq.fused_attention_packed(Q, cache)
+    big = (kv_input((1, 2, 1, 128), torch.float32, 7) * 1e7).to(dt).to(DEV)
+    cache.V.RANGE_CHECK_EVERY = 3
+    for i in range(3):
+        q.append(cache, x[:, :, i:i + 1], big if i == 0 else x[:, :, i:i + 1], 0)
+    assert cache.V.wide_range and not cache.K.wide_range
+    O = hqmq.fused_attention_packed(Q, cache)
+    assert torch.isfinite(O.float()).all() and float(O.float().abs().max()) > 10 * float(base.float().abs().max())
+    assert torch.equal(O, hqmq.fused_attention_packed(Q, cache, force_generic=True))
