@@ -165,7 +165,14 @@ constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chu
 constexpr int kFlagsTabMax = (kQOffset - kVTabOffset) / 8;      // codewords the V slot of the outlier variants holds
 static_assert(kFlagsTabMax * 8 + kVTabOffset == kQOffset && kFlagsTabMax == 4608, "V table slot of the outlier variants");
 constexpr int kSelOffset = kQOffset + 4096;        // outlier variants: nine rows of eight fp16, row r < 8 = unit vector r, row 8 = 0
-constexpr int kAuxTabOffset = 36864;        // s24_r3 only (K table <= 8 KB): 256 rows of 16 bytes, see decode_chunks
+constexpr int kAuxTabOffset = 36864;        // s192_r6: 64 dwords with the high radius bits of a pair of chunks, see gather_chunks
+// s24_r3 (13-bit codes, K <= 1024, qmax = 7): the tables are kept multiplied out, entry [rq][idx] = codeword * rq at byte
+// (rq << 10 | idx) * 8, so that the 13-bit code is the table index and a decode is one gather (no radius arithmetic).
+constexpr int kPsTabBytes = 8 * 1024 * 8;   // 64 KB per tensor
+constexpr bool is_prescaled(int CPL, int MB, int AB, int IB) { return CPL == 8 && MB == 12 && AB == 1 && IB == 10; }
+constexpr int vtab_offset(bool ps) { return ps ? kPsTabBytes : kVTabOffset; }
+constexpr int q_offset(bool ps) { return ps ? 2 * kPsTabBytes : kQOffset; }
+constexpr int sel_offset(bool ps) { return q_offset(ps) + 4096; }
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
@@ -253,25 +260,15 @@ __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t 
         }
     } else if constexpr (MB == 12 && AB == 1 && IB == 10 && CPL == 8) {
         static_assert(!F8, "the float8 table variants exist for 16-bit main fields");
-        // s24_r3: eight 12-bit fields (idx in the low 10 bits, the low two radius bits above) in three dwords
-        // and one aux byte with the eight high radius bits.  The aux byte indexes a 256-entry LDS table whose row
-        // holds, per pair of chunks, the two high radius bits at bits 2 and 18 and the 0x6400 fp16 magic.
-        const uint4v ax = *(lds_u4_ptr)(uintptr_t)(kAuxTabOffset + (aux & 0xffu) * 16u);
-        const uint32_t axs[4] = {ax[0], ax[1], ax[2], ax[3]};
+        // s24_r3, tables multiplied out (see kPsTabBytes): eight 12-bit fields (idx in the low 10 bits, the low two
+        // radius bits above) in three dwords and one aux byte with the eight high radius bits; field | aux bit << 12 is
+        // the table index.  No radius arithmetic: r stays unused.
         const uint32_t w0 = w[0], w1 = w[1], w2 = w[2];
-        constexpr uint32_t M = 0x1ff8u;
+        constexpr uint32_t M = 0x7ff8u;
         const uint32_t ad[8] = {(w0 << 3) & M, (w0 >> 9) & M, __builtin_amdgcn_alignbit(w1, w0, 21) & M, (w1 >> 1) & M,
                                 (w1 >> 13) & M, __builtin_amdgcn_alignbit(w2, w1, 25) & M, (w2 >> 5) & M, (w2 >> 17) & M};
 #pragma unroll
-        for (int j = 0; j < 8; j++) g[j] = gather8<TAB_OFF>(ad[j]);
-        const uint32_t lo2[8] = {__builtin_amdgcn_ubfe(w0, 10, 2), __builtin_amdgcn_ubfe(w0, 22, 2), __builtin_amdgcn_ubfe(w1, 2, 2),
-                                 __builtin_amdgcn_ubfe(w1, 14, 2), __builtin_amdgcn_ubfe(w1, 26, 2), __builtin_amdgcn_ubfe(w2, 6, 2),
-                                 __builtin_amdgcn_ubfe(w2, 18, 2), w2 >> 30};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t t = (lo2[2 * i] | (lo2[2 * i + 1] << 16)) | axs[i];
-            r[i] = __builtin_bit_cast(half2v, t) - k1024;
-        }
+        for (int j = 0; j < 8; j++) g[j] = gather8<TAB_OFF>(((aux << (15 - j)) & 0x8000u) | ad[j]);
     } else {
         static_assert(!F8, "the float8 table variants exist for the layouts with compile-time index widths");
 #pragma unroll
@@ -283,10 +280,10 @@ __device__ __forceinline__ void gather_chunks(const uint32_t (&w)[NW], uint32_t 
         }
     }
 }
-template <int CPL>
+template <int CPL, bool PS = false>
 __device__ __forceinline__ void scale_chunks(const half4 (&g)[CPL], const half2v (&r)[CPL / 2], half4 (&a)[CPL]) {
 #pragma unroll
-    for (int j = 0; j < CPL; j++) a[j] = g[j] * r[j >> 1][j & 1];
+    for (int j = 0; j < CPL; j++) a[j] = PS ? g[j] : g[j] * r[j >> 1][j & 1];
 }
 
 __device__ __forceinline__ half8 cat8(half4 x, half4 y) { return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7); }
@@ -332,7 +329,9 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     constexpr bool kBatchGathers = false;       // see half_step: measured, no gain on any shape (178 against 157 registers)
     constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
-    uint2 *ktab = lds_tab, *vtab = lds_tab + kVTabOffset / 8;
+    constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
+    constexpr int VTAB = vtab_offset(PS), QOFF = q_offset(PS), SELOFF = sel_offset(PS);
+    uint2 *ktab = lds_tab, *vtab = lds_tab + VTAB / 8;
     touch_kernargs();
 
     // blocks are dispatched in grid order: batch_order lists the sequences in the order they should start
@@ -509,13 +508,29 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     for (int e = 0; e < 4; e++) ident_bf[e] = (short)((4 * grp + e) == col ? 0x3F80 : 0);
 
     {
+        if constexpr (PS) {
+            // tables multiplied out: codeword * rq for rq = 0..7 at (rq << 10 | idx) * 8 (K <= 1024: FU * NT pairs cover it)
 #pragma unroll
-        for (int u = 0; u < FU; u++) {
-            const int k = threadIdx.x + u * NT;
-            if (k < Kk2) store_pair<DT, F8>(ktab, k, tk[u]);
-            if (k < Kv2) store_pair<DT, F8>(vtab, k, tv[u]);
+            for (int u = 0; u < FU; u++) {
+                const int k = threadIdx.x + u * NT;
+                const uint4v hk = pair_to_half<DT>(tk[u]), hv = pair_to_half<DT>(tv[u]);
+#pragma unroll
+                for (int rq = 0; rq < 8; rq++) {
+                    const half2v f = half2v{(_Float16)(float)rq, (_Float16)(float)rq};
+                    auto mul = [&](uint32_t w) { return __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, w) * f); };
+                    if (k < Kk2) reinterpret_cast<uint4v *>(ktab)[rq * 512 + k] = uint4v{mul(hk[0]), mul(hk[1]), mul(hk[2]), mul(hk[3])};
+                    if (k < Kv2) reinterpret_cast<uint4v *>(vtab)[rq * 512 + k] = uint4v{mul(hv[0]), mul(hv[1]), mul(hv[2]), mul(hv[3])};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < FU; u++) {
+                const int k = threadIdx.x + u * NT;
+                if (k < Kk2) store_pair<DT, F8>(ktab, k, tk[u]);
+                if (k < Kv2) store_pair<DT, F8>(vtab, k, tv[u]);
+            }
+            if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT, F8>(ktab, ksrc, Kk2, vtab, vsrc, Kv2, FU * NT);
         }
-        if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT, F8>(ktab, ksrc, Kk2, vtab, vsrc, Kv2, FU * NT);
     }
     // Plain variants keep two half-steps in flight.  The second one is requested only now, when the table loads
     // have come back: requested at the start it would queue in front of them and delay the whole block.
@@ -530,7 +545,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         // the selector rows carry qmax instead of 1: the gathered probabilities come out scaled for the verbatim
         // chunks (whose 1 / qmax is applied with everything else in the epilogue) at no cost
         const uint32_t one = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(float)p.qmax);
-        reinterpret_cast<uint32_t *>(lds_tab)[kSelOffset / 4 + w] = (row < 8 && (row >> 1) == d) ? one << (16 * (row & 1)) : 0u;
+        reinterpret_cast<uint32_t *>(lds_tab)[SELOFF / 4 + w] = (row < 8 && (row >> 1) == d) ? one << (16 * (row & 1)) : 0u;
     }
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
@@ -543,24 +558,14 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 q8 = uint4v{lo.x, lo.y, hi.x, hi.y};
             }
             const int c0 = grp * CPL + 2 * jj;
-            lds_tab[kQOffset / 8 + c0 * 16 + col] = uint2{q8[0], q8[1]};
-            lds_tab[kQOffset / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
+            lds_tab[QOFF / 8 + c0 * 16 + col] = uint2{q8[0], q8[1]};
+            lds_tab[QOFF / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
         }
     }
     if constexpr (MB == 16 && AB == 3 && IB == 13) {
         if (threadIdx.x < 64) {
             const uint32_t b6 = threadIdx.x;
             reinterpret_cast<uint32_t *>(lds_tab)[kAuxTabOffset / 4 + b6] = ((b6 & 7u) << 3) | ((b6 >> 3) << 19) | 0x64006400u;
-        }
-    }
-    if constexpr (MB == 12 && AB == 1 && IB == 10) {
-        if (threadIdx.x < 256) {
-            const uint32_t b8 = threadIdx.x;
-            uint32_t row[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) row[i] = (((b8 >> (2 * i)) & 1u) << 2) | (((b8 >> (2 * i + 1)) & 1u) << 18) | 0x64006400u;
-            lds_tab[kAuxTabOffset / 8 + 2 * b8] = uint2{row[0], row[1]};
-            lds_tab[kAuxTabOffset / 8 + 2 * b8 + 1] = uint2{row[2], row[3]};
         }
     }
     __syncthreads();
@@ -603,8 +608,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const int e0 = bs + 2 * grp;
         const uint32_t c0 = cc & (uint32_t)(n - 1), c1 = (cc >> 16) & (uint32_t)(n - 1);
         const int r0 = (cc >> 8) & 15, r1 = (cc >> 24) & 15;
-        const uint2 q0r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(kQOffset + c0 * 128u + (uint32_t)col * 8u));
-        const uint2 q1r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(kQOffset + c1 * 128u + (uint32_t)col * 8u));
+        const uint2 q0r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c0 * 128u + (uint32_t)col * 8u));
+        const uint2 q1r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c1 * 128u + (uint32_t)col * 8u));
         const uint2 zero_u2 = uint2{0u, 0u};
         half4 h0 = zero_h4, h1 = zero_h4;
         if constexpr (!kBfEntries) { h0 = chunk_to_half<DT>(x[0]); h1 = chunk_to_half<DT>(x[1]); }
@@ -660,7 +665,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const uint32_t ch = cc & (uint32_t)(n - 1), t = (cc >> 8) & 15u;
         const uint32_t slot = (e >= off[1] ? 4u : 0u) + (t & 3u);             // position among the row group's 8 tokens
         const bool mine = ok && (int)(t >> 2) == grp;
-        const uint4v sel = *(lds_u4_ptr)(uintptr_t)(kSelOffset + (mine ? slot : 8u) * 16u);
+        const uint4v sel = *(lds_u4_ptr)(uintptr_t)(SELOFF + (mine ? slot : 8u) * 16u);
         const half4 pg = pack4(__builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0));
         half4 h = zero_h4;
         if constexpr (!kBfEntries) h = chunk_to_half<DT>(x);
@@ -711,7 +716,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         for (int u = 0; u < 2; u++) {
             half4 a[CPL];
             if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, 0, F8>(h.kw[u], AB ? h.kaux[u] : 0u, idx_bits, gk[u], rk[u]);
-            scale_chunks<CPL>(gk[u], rk[u], a);
+            scale_chunks<CPL, PS>(gk[u], rk[u], a);
 #pragma unroll
             for (int cgi = 0; cgi < NCG; cgi++) {
                 float4v s = zero4;
@@ -729,7 +734,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         half2v rv[2][CPL / 2];
         if constexpr (kBatchGathers) {
 #pragma unroll
-            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            for (int u = 0; u < 2; u++) gather_chunks<CPL, MB, AB, IB, NW, VTAB, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
         // ---- mask (boundary half-steps only), online softmax, per column group ----
@@ -782,8 +787,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         half4 av[2][CPL];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, kVTabOffset, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
-            scale_chunks<CPL>(gv[u], rv[u], av[u]);
+            if constexpr (!kBatchGathers) gather_chunks<CPL, MB, AB, IB, NW, VTAB, F8>(h.vw[u], AB ? h.vaux[u] : 0u, idx_bits, gv[u], rv[u]);
+            scale_chunks<CPL, PS>(gv[u], rv[u], av[u]);
         }
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
@@ -903,7 +908,8 @@ template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves, int NCG 
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
     if (NCG > 1) grid.y = (grid.y + NCG - 1) / NCG;
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
-    size_t shmem = flags ? (size_t)kSelOffset + 9 * 16 : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
+    size_t shmem = flags ? (size_t)sel_offset(PS) + 9 * 16 : PS ? (size_t)2 * kPsTabBytes : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
     const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);     // WV >= the wavefronts actually launched
     if (shmem < merge) shmem = merge;
     constexpr int WF = CPL == 4 ? WV : kFastWaves;      // outlier variants fit three wavefronts per SIMD only at d_h 64
