@@ -21,6 +21,8 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef const uint2 __attribute__((address_space(3))) *lds_u2_ptr;
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint4v uint4v_a8 __attribute__((aligned(8)));         // a 16-byte vector at an 8-byte aligned address
+typedef uint32_t uint32_a2 __attribute__((aligned(2)));       // a dword at a 2-byte aligned address
 
 template <int DT>
 __device__ __forceinline__ half4 chunk_to_half(uint2 w) {
@@ -164,7 +166,6 @@ constexpr int kVTabOffset = 40960;          // bytes; room for 5120 K codewords 
 constexpr int kQOffset = kVTabOffset + 36864;     // outlier variants: Q as [chunk][column] fp16 chunks, after the V table
 constexpr int kFlagsTabMax = (kQOffset - kVTabOffset) / 8;      // codewords the V slot of the outlier variants holds
 static_assert(kFlagsTabMax * 8 + kVTabOffset == kQOffset && kFlagsTabMax == 4608, "V table slot of the outlier variants");
-constexpr int kSelOffset = kQOffset + 4096;        // outlier variants: nine rows of eight fp16, row r < 8 = unit vector r, row 8 = 0
 constexpr int kAuxTabOffset = 36864;        // s192_r6: 64 dwords with the high radius bits of a pair of chunks, see gather_chunks
 // s24_r3 (13-bit codes, K <= 1024, qmax = 7): the tables are kept multiplied out, entry [rq][idx] = codeword * rq at byte
 // (rq << 10 | idx) * 8, so that the 13-bit code is the table index and a decode is one gather (no radius arithmetic).
@@ -172,7 +173,7 @@ constexpr int kPsTabBytes = 8 * 1024 * 8;   // 64 KB per tensor
 constexpr bool is_prescaled(int CPL, int MB, int AB, int IB) { return CPL == 8 && MB == 12 && AB == 1 && IB == 10; }
 constexpr int vtab_offset(bool ps) { return ps ? kPsTabBytes : kVTabOffset; }
 constexpr int q_offset(bool ps) { return ps ? 2 * kPsTabBytes : kQOffset; }
-constexpr int sel_offset(bool ps) { return q_offset(ps) + 4096; }
+constexpr int sel_offset(bool ps) { return q_offset(ps) + 4096; }      // nine rows of eight fp16: row r < 8 = qmax times unit vector r, row 8 = 0
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef const uint4v __attribute__((address_space(3))) *lds_u4_ptr;
@@ -415,7 +416,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     const char *v_side = FLAGS ? (const char *)p.Vc.sideband + (size_t)bh * p.Vc.sb_cap * 8 : nullptr;
     const char *k_coord = FLAGS ? (const char *)p.Kc.sb_coord + (size_t)bh * p.Kc.sb_cap * 2 : nullptr;
     const char *v_coord = FLAGS ? (const char *)p.Vc.sb_coord + (size_t)bh * p.Vc.sb_cap * 2 : nullptr;
-    const uint32_t k_cap1 = FLAGS ? (uint32_t)(p.Kc.sb_cap - 1) : 0u, v_cap1 = FLAGS ? (uint32_t)(p.Vc.sb_cap - 1) : 0u;
+    const uint32_t v_cap1 = FLAGS ? (uint32_t)(p.Vc.sb_cap - 1) : 0u;
+    const uint32_t k_cap2 = FLAGS ? (uint32_t)(p.Kc.sb_cap - 2) : 0u;        // sb_cap >= 2 is checked at launch
 
     auto load_super = [&](int t0, FastTile<NW, AB, FLAGS, NH> &s) {
         // in the order the half-steps consume them: K, then V, of tokens 0..31, then the same of tokens 32..63
@@ -453,14 +455,30 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             qf[cgi][j] = cat8(lo, hi);
         }
     }
+    // Tile offsets of one half-step, in two parts.  The loads (of wave-uniform addresses) are requested two half-steps
+    // ahead; their clamping, which makes the values scalar, happens only when flags_ready has let them through at
+    // the end of a half-step: placed right behind the loads it would wait for them with every later load in flight.
     auto load_flags = [&](int th, FlagTile &f) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const int tc = min((th >> 4) + i, tiles_cap1);
+            f.koff[i] = k_toff[tc];
+            f.voff[i] = v_toff[tc];
+        }
+    };
+    auto flags_ready = [&](int th, FlagTile &f) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            asm volatile("" : "+v"(f.koff[i]), "+v"(f.voff[i]));
+            f.koff[i] = __builtin_amdgcn_readfirstlane(f.koff[i]);       // the same value in every lane: scalar from here on
+            f.voff[i] = __builtin_amdgcn_readfirstlane(f.voff[i]);
+        }
         // tiles not written yet hold INT32_MAX, and so does the slot after the last tile: the count bounds them
 #pragma unroll
         for (int i = 0; i < 3; i++) {
-            const int ti = (th >> 4) + i, tc = min(ti, tiles_cap1);
-            const int kv = k_toff[tc], vv = v_toff[tc];
-            f.koff[i] = min(ti <= tiles_cap1 ? kv : 0x7fffffff, k_count);
-            f.voff[i] = min(ti <= tiles_cap1 ? vv : 0x7fffffff, v_count);
+            const bool in = (th >> 4) + i <= tiles_cap1;
+            f.koff[i] = min(in ? f.koff[i] : 0x7fffffff, k_count);
+            f.voff[i] = min(in ? f.voff[i] : 0x7fffffff, v_count);
         }
         // a tile has at most 16 n entries: bounds the walk if the caller's offsets are inconsistent
 #pragma unroll
@@ -494,7 +512,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const int t_first = min(t_begin, (int)p.t_cap - 32);
         if (FLAGS) load_flags(t_first, f0);
         load_super(t_first, cur);
-        if (FLAGS) load_flags(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);
+        if (FLAGS) load_flags(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);        // made ready below
     }
 
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
@@ -589,56 +607,71 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // flag is read: a batch of eight entries is the reduction dimension of one MFMA per tile,
     //   so[token][column] += sum over entries e of the batch, i < 4:  [token(e) == token] x_e[i] * Q[column][4 chunk(e) + i],
     // A = the lane's two entries where their token is the lane's row (else zero), B = the Q chunks they meet (LDS).
+    // The lane's two entries are neighbours in the list: one 16-byte load of the chunks (8-byte aligned) and one 4-byte
+    // load of the coordinates (2-byte aligned), at 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked
+    // at launch).  The pair is clamped to the last pair of the list's storage: an entry that is the very last slot of
+    // a full list then arrives in the upper half.  (A wave-uniform branch to an unclamped variant measures slower.)
     auto k_load = [&](int bs, uint2 (&x)[2], uint32_t &cc) {
-        // 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked at launch)
-        const uint32_t e0 = min((uint32_t)bs + 2u * (uint32_t)grp, k_cap1), e1 = min(e0 + 1u, k_cap1);
-        x[0] = *reinterpret_cast<const uint2 *>(k_side + e0 * 8u);
-        x[1] = *reinterpret_cast<const uint2 *>(k_side + e1 * 8u);
-        cc = (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e0 * 2u) | (uint32_t)*reinterpret_cast<const uint16_t *>(k_coord + e1 * 2u) << 16;
+        const uint32_t e0 = (uint32_t)bs + 2u * (uint32_t)grp, ec = min(e0, k_cap2);
+        const uint4v X = *reinterpret_cast<const uint4v_a8 *>(k_side + ec * 8u);
+        const uint32_t C = *reinterpret_cast<const uint32_a2 *>(k_coord + ec * 2u);
+        const bool up = e0 > k_cap2;
+        x[0] = uint2{up ? X[2] : X[0], up ? X[3] : X[1]};
+        x[1] = uint2{X[2], X[3]};
+        cc = up ? C >> 16 : C;
     };
     auto k_issue = [&](const FlagTile &f, KPre<kKPre> &k) {
 #pragma unroll
         for (int i = 0; i < 3; i++) k.off[i] = f.koff[i];
 #pragma unroll
-        for (int bq = 0; bq < kKPre; bq++) {
-            k_load(k.off[0] + 8 * bq, k.x[bq], k.cc[bq]);
-        }
+        for (int bq = 0; bq < kKPre; bq++) k_load(k.off[0] + 8 * bq, k.x[bq], k.cc[bq]);
     };
-    auto k_batch = [&](const int (&off)[3], int bs, const uint2 (&x)[2], uint32_t cc, float4v (&so)[2]) {
-        const int e0 = bs + 2 * grp;
+    // the Q chunks the lane's two entries meet (B operand rows), read from LDS well before the batch's MFMAs
+    auto k_qrows = [&](uint32_t cc, uint2 (&q)[2]) {
         const uint32_t c0 = cc & (uint32_t)(n - 1), c1 = (cc >> 16) & (uint32_t)(n - 1);
-        const int r0 = (cc >> 8) & 15, r1 = (cc >> 24) & 15;
-        const uint2 q0r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c0 * 128u + (uint32_t)col * 8u));
-        const uint2 q1r = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c1 * 128u + (uint32_t)col * 8u));
+        q[0] = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c0 * 128u + (uint32_t)col * 8u));
+        q[1] = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c1 * 128u + (uint32_t)col * 8u));
+    };
+    auto k_batch = [&](const int (&off)[3], int bs, const uint2 (&x)[2], uint32_t cc, const uint2 (&q)[2], float4v (&so)[2]) {
+        const int e0 = bs + 2 * grp;
+        // the row of the half-step (0..31) an entry belongs to; 64 for a slot behind the half-step's entries
+        const uint32_t k0 = e0 < off[2] ? ((cc >> 8) & 15u) + (e0 >= off[1] ? 16u : 0u) : 64u;
+        const uint32_t k1 = e0 + 1 < off[2] ? ((cc >> 24) & 15u) + (e0 + 1 >= off[1] ? 16u : 0u) : 64u;
         const uint2 zero_u2 = uint2{0u, 0u};
         half4 h0 = zero_h4, h1 = zero_h4;
         if constexpr (!kBfEntries) { h0 = chunk_to_half<DT>(x[0]); h1 = chunk_to_half<DT>(x[1]); }
-        const half8 qq = cat8(__builtin_bit_cast(half4, q0r), __builtin_bit_cast(half4, q1r));
+        const half8 qq = cat8(__builtin_bit_cast(half4, q[0]), __builtin_bit_cast(half4, q[1]));
+        // both tiles, no branch: the matrix unit is idle here and a skipped MFMA saves less than its test costs
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            if (bs < off[u + 1] && bs + 8 > off[u]) {        // wave-uniform: the batch meets tile u
-                const bool v0 = e0 >= off[u] && e0 < off[u + 1] && r0 == col;
-                const bool v1 = e0 + 1 >= off[u] && e0 + 1 < off[u + 1] && r1 == col;
-                if constexpr (kBfEntries) {
-                    const uint2 a0 = v0 ? x[0] : zero_u2, a1 = v1 ? x[1] : zero_u2;
-                    so[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, uint4v{a0.x, a0.y, a1.x, a1.y}),
-                                                                    __builtin_bit_cast(bf16x8, uint4v{q0r.x, q0r.y, q1r.x, q1r.y}),
-                                                                    so[u], 0, 0, 0);
-                } else {
-                    so[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(v0 ? h0 : zero_h4, v1 ? h1 : zero_h4), qq, so[u], 0, 0, 0);
-                }
+            const bool v0 = k0 == (uint32_t)(col + 16 * u), v1 = k1 == (uint32_t)(col + 16 * u);
+            if constexpr (kBfEntries) {
+                const uint2 a0 = v0 ? x[0] : zero_u2, a1 = v1 ? x[1] : zero_u2;
+                so[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, uint4v{a0.x, a0.y, a1.x, a1.y}),
+                                                                __builtin_bit_cast(bf16x8, uint4v{q[0].x, q[0].y, q[1].x, q[1].y}),
+                                                                so[u], 0, 0, 0);
+            } else {
+                so[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(v0 ? h0 : zero_h4, v1 ? h1 : zero_h4), qq, so[u], 0, 0, 0);
             }
         }
     };
-    auto k_apply = [&](const KPre<kKPre> &k, float4v (&so)[2]) {
+    struct KRows {
+        uint2 q[kKPre][2];
+    };
+    auto k_prepare = [&](const KPre<kKPre> &k, KRows &r) {
+#pragma unroll
+        for (int bq = 0; bq < kKPre; bq++) k_qrows(k.cc[bq], r.q[bq]);
+    };
+    auto k_apply = [&](const KPre<kKPre> &k, const KRows &r, float4v (&so)[2]) {
 #pragma unroll
         for (int bq = 0; bq < kKPre; bq++)
-            if (k.off[0] + 8 * bq < k.off[2]) k_batch(k.off, k.off[0] + 8 * bq, k.x[bq], k.cc[bq], so);
+            if (k.off[0] + 8 * bq < k.off[2]) k_batch(k.off, k.off[0] + 8 * bq, k.x[bq], k.cc[bq], r.q[bq], so);
         for (int bs = k.off[0] + 8 * kKPre; bs < k.off[2]; bs += 8) {      // more than the prefetched batches: rare
-            uint2 x[2];
+            uint2 x[2], q[2];
             uint32_t cc;
             k_load(bs, x, cc);
-            k_batch(k.off, bs, x, cc, so);
+            k_qrows(cc, q);
+            k_batch(k.off, bs, x, cc, q, so);
         }
     };
     // V side, also from the entry list, sixteen entries of the half-step per batch (lane 16 * grp + col holds
@@ -659,40 +692,51 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
         for (int bq = 0; bq < kVPre; bq++) v_load(v.off[0] + 16 * bq, v.x[bq], v.cc[bq]);
     };
-    auto v_batch = [&](const int (&off)[3], int bs, uint2 x, uint32_t cc, half8 ppo) {
+    // the selector row of the lane's entry (A operand of the MFMA that gathers the probabilities), read ahead of use
+    auto v_sel = [&](const int (&off)[3], int bs, uint32_t cc) {
         const int e = bs + col;
-        const bool ok = e < off[2];
-        const uint32_t ch = cc & (uint32_t)(n - 1), t = (cc >> 8) & 15u;
+        const uint32_t t = (cc >> 8) & 15u;
         const uint32_t slot = (e >= off[1] ? 4u : 0u) + (t & 3u);             // position among the row group's 8 tokens
-        const bool mine = ok && (int)(t >> 2) == grp;
-        const uint4v sel = *(lds_u4_ptr)(uintptr_t)(SELOFF + (mine ? slot : 8u) * 16u);
+        const bool mine = e < off[2] && (int)(t >> 2) == grp;
+        return *(lds_u4_ptr)(uintptr_t)(SELOFF + (mine ? slot : 8u) * 16u);
+    };
+    auto v_batch = [&](const int (&off)[3], int bs, uint2 x, uint32_t cc, uint4v sel, half8 ppo) {
+        const int e = bs + col;
+        const uint32_t ch = cc & (uint32_t)(n - 1);
         const half4 pg = pack4(__builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sel), ppo, zero4, 0, 0, 0));
         half4 h = zero_h4;
         if constexpr (!kBfEntries) h = chunk_to_half<DT>(x);
-        const bool owner = ok && (int)(ch / CPL) == grp;
+        const bool owner = e < off[2] && (int)(ch / CPL) == grp;
         const int jq = (int)(ch % CPL);
+        // every chunk position, no test whether the batch meets it: straight-line code measures faster than skipping
+        // the positions without an entry (the matrix unit is idle here, and a wave-uniform branch costs more than two MFMAs)
 #pragma unroll
         for (int j = 0; j < CPL; j++) {
             const bool mj = owner && jq == j;
-            if (__builtin_amdgcn_ballot_w64(mj) != 0) {
-                float4v tr;
-                if constexpr (kBfEntries)
-                    tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, mj ? x : uint2{0u, 0u}), ident_bf, zero4, 0, 0, 0);
-                else
-                    tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
-            }
+            float4v tr;
+            if constexpr (kBfEntries)
+                tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, mj ? x : uint2{0u, 0u}), ident_bf, zero4, 0, 0, 0);
+            else
+                tr = __builtin_amdgcn_mfma_f32_16x16x16f16(mj ? h : zero_h4, ident, zero4, 0, 0, 0);
+            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(pack4(tr), pg, acc[0][j], 0, 0, 0);
         }
     };
-    auto v_apply = [&](const VPre<kVPre> &v, half8 ppo) {
+    struct VSel {
+        uint4v s[kVPre];
+    };
+    auto v_prepare = [&](const VPre<kVPre> &v, VSel &r) {
+#pragma unroll
+        for (int bq = 0; bq < kVPre; bq++) r.s[bq] = v_sel(v.off, v.off[0] + 16 * bq, v.cc[bq]);
+    };
+    auto v_apply = [&](const VPre<kVPre> &v, const VSel &r, half8 ppo) {
 #pragma unroll
         for (int bq = 0; bq < kVPre; bq++)
-            if (v.off[0] + 16 * bq < v.off[2]) v_batch(v.off, v.off[0] + 16 * bq, v.x[bq], v.cc[bq], ppo);
+            if (v.off[0] + 16 * bq < v.off[2]) v_batch(v.off, v.off[0] + 16 * bq, v.x[bq], v.cc[bq], r.s[bq], ppo);
         for (int bs = v.off[0] + 16 * kVPre; bs < v.off[2]; bs += 16) {     // more than the prefetched batches: rare
             uint2 x;
             uint32_t cc;
             v_load(bs, x, cc);
-            v_batch(v.off, bs, x, cc, ppo);
+            v_batch(v.off, bs, x, cc, v_sel(v.off, bs, cc), ppo);
         }
     };
 
@@ -701,7 +745,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // value from the sideband contributes.
     auto half_step = [&](const HalfTile<NW, AB, FLAGS> &h, int th, const KPre<kKPre> &kc, const VPre<kVPre> &vc) {
         float4v sT[NCG][2], so[2] = {zero4, zero4};
-        if (FLAGS) k_apply(kc, so);
+        // the LDS operands of the outlier batches are requested first and used after the main products
+        KRows kr;
+        VSel vr;
+        if constexpr (FLAGS) {
+            k_prepare(kc, kr);
+            v_prepare(vc, vr);
+        }
         // every gather of the 32 K tokens is requested before the first one is used: the wavefront waits for LDS
         // once per half-step and tensor, not once per pair of chunks
         // (the variants that have no registers to spare keep the compiler's own interleaving of gathers and multiplies)
@@ -723,11 +773,20 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
                 for (int jj = 0; jj < CPL / 2; jj++)
                     s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[cgi][jj], s, 0, 0, 0);
+                if constexpr (!FLAGS) {
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, FLAGS ? so[u][e] * qmaxf : 0.f);
+                    for (int e = 0; e < 4; e++) s[e] = scaled<DT>(s[e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, 0.f);
+                }
                 sT[cgi][u] = s;
             }
+        }
+        if constexpr (FLAGS) {
+            k_apply(kc, kr, so);
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    sT[0][u][e] = scaled<DT>(sT[0][u][e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, so[u][e] * qmaxf);
         }
         // the V gathers fly while the softmax below keeps the vector unit busy
         half4 gv[2][CPL];
@@ -798,7 +857,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
             for (int cgi = 0; cgi < NCG; cgi++) acc[cgi][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pp[cgi], acc[cgi][j], 0, 0, 0);
         }
-        if (FLAGS) v_apply(vc, cat8(pTo[0], pTo[1]));
+        if constexpr (FLAGS) v_apply(vc, vr, cat8(pTo[0], pTo[1]));
     };
 
     // sideband requests of one half-step
@@ -808,7 +867,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     };
     KPre<kKPre> kc = {};
     VPre<kVPre> vc = {};
-    if (FLAGS && t_begin < t_end) issue_all(f0, kc, vc);
+    if constexpr (FLAGS) {
+        const int t_first = min(t_begin, (int)p.t_cap - 32);
+        flags_ready(t_first, f0);
+        flags_ready(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);
+        if (t_begin < t_end) issue_all(f0, kc, vc);
+    }
 
     if constexpr (!FLAGS) {
         // ring of three tile buffers, every load unconditional (past the end the current tile is requested again)
@@ -841,7 +905,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             // tile offsets two steps ahead, sideband entries one step ahead (their offsets were requested a step
             // ago); past the end the current tile is requested again
             load_super(more ? t0 + STEP : t0, nxt);
-            load_flags(more2 ? t0 + 2 * STEP : t0, f2);
+            load_flags(more2 ? t0 + 2 * STEP : t0, f2);           // made ready at the end of this half-step
             issue_all(f1, kn, vn);
         } else if (more) {
             load_super(t0 + STEP, nxt);
@@ -853,6 +917,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             if (FLAGS) {
                 kc = kn;
                 vc = vn;
+                flags_ready(more2 ? t0 + 2 * STEP : t0, f2);
                 f1 = f2;
             }
         }
