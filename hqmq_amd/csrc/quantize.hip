@@ -21,6 +21,7 @@
 //
 // Compiled with -ffp-contract=off; fused multiply-adds are written explicitly.
 #include "common.h"
+#include <type_traits>
 
 namespace hqmq {
 
@@ -226,21 +227,51 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             // for every block, lane i holds column i), B = the lane's own direction, D = its rotated chunk.
             const half4 ub = half4{(_Float16)us[0], (_Float16)us[1], (_Float16)us[2], (_Float16)us[3]};
             const uint2 *acol = rot + (tid & 3);
+            // The scan runs in blocks of 32 secondaries whose scores stay in registers.  Only the running maximum is
+            // kept inside a block; at its end the secondaries within the margin of the maximum so far become a bit mask
+            // (a compare and an add-with-carry each) and go into the list of the re-score below.  A maximum that has
+            // moved up by more than the margin during the block leaves everything listed before more than the margin
+            // below the final maximum: the list starts over.
+            const int iters = (S + slots - 1) / slots;          // of the slot with the most secondaries (wave-uniform)
             uint2 a_next = acol[4 * min(s_first, S - 1)];
-            for (int s = s_first; s < S; s += slots) {
-                const half4 am = __builtin_bit_cast(half4, a_next);
-                a_next = acol[4 * min(s + slots, S - 1)];       // the next column is on its way during this one
-                const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                const float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
-                // kept: within the margin of the running maximum.  A score that beats the old maximum by more than the
-                // margin leaves everything kept so far more than the margin below the final maximum: the list starts
-                // over, which keeps it at the true candidates instead of every record of the scan.
-                if (b2 + margin2 >= m2) {
-                    if (b2 - margin2 > m2) cnt = 0;
-                    if (cnt < kSCap) slist[cnt][tid] = (uint16_t)s;
+            auto scan_block = [&](int i0, auto tail) -> uint32_t {
+                float b2v[32];
+#pragma unroll
+                for (int i = 0; i < 32; i++) {
+                    const int sn = s_first + (i0 + i + 1) * slots;
+                    const half4 am = __builtin_bit_cast(half4, a_next);
+                    // the next column is on its way during this one; inside a whole block it exists, so its address is
+                    // the block's base plus a constant
+                    a_next = (decltype(tail)::value || i == 31) ? acol[4 * min(sn, S - 1)] : acol[4 * sn];
+                    const float4v vv = __builtin_amdgcn_mfma_f32_4x4x4f16(am, ub, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
+                    if (decltype(tail)::value && sn - slots >= S) b2 = -INFINITY;      // behind the slot's last secondary
+                    b2v[i] = b2;
+                    asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
+                }
+                const float thr = m2 - margin2;
+                uint32_t word = 0u;
+#pragma unroll
+                for (int i = 31; i >= 0; i--)       // word = 2 word + (score >= thr): iteration i ends up in bit i
+                    asm("v_cmp_ge_f32_e32 vcc, %1, %2\n\tv_addc_co_u32_e32 %0, vcc, %0, %0, vcc" : "+v"(word) : "v"(b2v[i]), "v"(thr) : "vcc");
+                if (decltype(tail)::value) {        // a slot whose secondaries end inside the block: only those count
+                    const int left = S - s_first - i0 * slots;
+                    const int valid = left <= 0 ? 0 : min((left + slots - 1) / slots, 32);
+                    word &= valid >= 32 ? ~0u : (1u << valid) - 1u;
+                }
+                return word;
+            };
+            for (int i0 = 0; i0 < iters; i0 += 32) {
+                const float m_before = m2;
+                const bool whole = (slots - 1) + (i0 + 31) * slots < S;     // every slot has all 32 secondaries of this block
+                uint32_t bits = whole ? scan_block(i0, std::false_type{}) : scan_block(i0, std::true_type{});
+                if (m_before < m2 - margin2) cnt = 0;
+                while (bits) {
+                    const int i = __builtin_ctz(bits);
+                    bits &= bits - 1u;
+                    if (cnt < kSCap) slist[cnt][tid] = (uint16_t)(s_first + (i0 + i) * slots);
                     cnt++;
                 }
-                asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
             }
         } else {
             for (int s = 0; s < S; s++) {
@@ -406,25 +437,49 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
         __syncthreads();
         const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
         const bool row_ok = active && writer && row >= 0 && row < a.t_cap;  // a bad pos[] must not write outside the plane
+        // one-bit planes (flags, a one-bit aux field) of tokens whose lanes sit side by side in a wavefront come
+        // straight from a ballot: the token's n bits are n / 8 whole bytes of it
+        const bool side_by_side = (n & (n - 1)) == 0 && n >= 8 && n <= 64;
+        const int lane_base = (tid & 63) / n * n;
+        const uint64_t aux_bits1 = __builtin_amdgcn_ballot_w64(((code_sh[tid] >> a.main_bits) & 1u) != 0u);
+        const uint64_t flag_bits1 = __builtin_amdgcn_ballot_w64(flagged);
         if (row_ok) {
             const size_t prow = ((size_t)b * a.H + h) * a.t_cap + row;
             const uint32_t *codes = code_sh + tok_local * n;
             if (a.main_plane) {
                 const int rb = (n * a.main_bits + 7) >> 3;
                 uint8_t *dst = a.main_plane + prow * rb;
-                if (a.main_bits == 16) reinterpret_cast<uint16_t *>(dst)[c] = (uint16_t)codes[c];   // one code per lane
-                else
+                if (a.main_bits == 16) {
+                    reinterpret_cast<uint16_t *>(dst)[c] = (uint16_t)codes[c];   // one code per lane
+                } else if (a.main_bits == 12 && !(n & 1)) {
+                    if (!(c & 1)) {                                             // two codes = three bytes
+                        const uint32_t two = (codes[c] & 0xfffu) | ((codes[c + 1] & 0xfffu) << 12);
+                        uint8_t *d = dst + (c >> 1) * 3;
+                        d[0] = (uint8_t)two;
+                        d[1] = (uint8_t)(two >> 8);
+                        d[2] = (uint8_t)(two >> 16);
+                    }
+                } else {
                     for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.main_bits, 0, byte);
+                }
             }
             if (a.aux_plane && a.aux_bits) {
                 const int rb = (n * a.aux_bits + 7) >> 3;
                 uint8_t *dst = a.aux_plane + prow * rb;
-                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.aux_bits, a.main_bits, byte);
+                if (a.aux_bits == 1 && side_by_side) {
+                    if (c < rb) dst[c] = (uint8_t)(aux_bits1 >> (lane_base + 8 * c));
+                } else {
+                    for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(codes, n, a.aux_bits, a.main_bits, byte);
+                }
             }
             if (a.flag_plane) {
                 const int rb = (n + 7) >> 3;
                 uint8_t *dst = a.flag_plane + prow * rb;
-                for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(mask_sh + tok_local * n, n, 1, 0, byte);
+                if (side_by_side) {
+                    if (c < rb) dst[c] = (uint8_t)(flag_bits1 >> (lane_base + 8 * c));
+                } else {
+                    for (int byte = c; byte < rb; byte += n) dst[byte] = gather_byte(mask_sh + tok_local * n, n, 1, 0, byte);
+                }
             }
             if (a.scale_plane && c == 0) D::store((ST *)a.scale_plane + prow, rm);
         }
@@ -485,9 +540,13 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(QParams a) {
 
 // The K and the V rows of one append in one launch (same shapes): blockIdx.z picks the tensor.  A single-token
 // append is latency-bound (32 lanes per block for a few microseconds), so the two run side by side for free.
+struct QPair {
+    QParams p[2];       // K, V
+};
+// (indexed in the kernel-argument segment: one set of scalar registers, not a select per field of two structs)
 template <class D, bool SPLIT>
-__global__ __launch_bounds__(kQThreads) void quantize_pair_kernel(QParams k, QParams v) {
-    quantize_body<D, 0, SPLIT>(blockIdx.z ? v : k);
+__global__ __launch_bounds__(kQThreads) void quantize_pair_kernel(QPair kv) {
+    quantize_body<D, 0, SPLIT>(kv.p[blockIdx.z]);
 }
 template <class D>
 __global__ __launch_bounds__(kQThreads) void quantize_split_kernel(QParams a) {
@@ -521,11 +580,11 @@ static int launch_quantize_pair(const QParams &k, const QParams &v, hipStream_t 
     size_t shmem = (size_t)k.S * 4 * sizeof(float) + (size_t)k.S * 4 * sizeof(uint2);
     if constexpr (sizeof(typename D::storage) == 2) {
         if (use_split<D>(k, 0) && use_split<D>(v, 0)) {
-            hipLaunchKernelGGL((quantize_pair_kernel<D, true>), grid, block, shmem, st, k, v);
+            hipLaunchKernelGGL((quantize_pair_kernel<D, true>), grid, block, shmem, st, QPair{{k, v}});
             return hip_status(hipGetLastError());
         }
     }
-    hipLaunchKernelGGL((quantize_pair_kernel<D, false>), grid, block, shmem, st, k, v);
+    hipLaunchKernelGGL((quantize_pair_kernel<D, false>), grid, block, shmem, st, QPair{{k, v}});
     return hip_status(hipGetLastError());
 }
 
