@@ -32,6 +32,34 @@ constexpr int kQThreads = 256;
 constexpr int kSCap = 32;  // candidate secondaries kept per lane
 constexpr int kKCap = 24;  // candidate codewords kept per lane
 
+// Maximum over groups of `n` neighbouring lanes (n a power of two up to 64), every lane of a group receiving it:
+// lane permutations inside the vector unit (quad, half-row and row mirrors, then the 16- and 32-lane row swaps).
+// The operands are ordinary numbers or -inf (no NaN), as unsigned bit patterns of non-negative floats order like the
+// values, the same routine serves both.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, false);
+}
+template <class T, class MAX>
+__device__ __forceinline__ T group_max(T x, int n, MAX mx) {
+    auto step = [&](uint32_t other) { x = mx(x, __builtin_bit_cast(T, other)); };
+    if (n >= 2) step(dpp_u32<0xB1>(__builtin_bit_cast(uint32_t, x)));       // quad_perm [1,0,3,2]
+    if (n >= 4) step(dpp_u32<0x4E>(__builtin_bit_cast(uint32_t, x)));       // quad_perm [2,3,0,1]
+    if (n >= 8) step(dpp_u32<0x141>(__builtin_bit_cast(uint32_t, x)));      // row_half_mirror
+    if (n >= 16) step(dpp_u32<0x140>(__builtin_bit_cast(uint32_t, x)));     // row_mirror
+    if (n >= 32) {
+        const uint32_t b = __builtin_bit_cast(uint32_t, x);
+        const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+        x = mx(__builtin_bit_cast(T, (uint32_t)r[0]), __builtin_bit_cast(T, (uint32_t)r[1]));
+    }
+    if (n >= 64) {
+        const uint32_t b = __builtin_bit_cast(uint32_t, x);
+        const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+        x = mx(__builtin_bit_cast(T, (uint32_t)r[0]), __builtin_bit_cast(T, (uint32_t)r[1]));
+    }
+    return x;
+}
+
 struct QParams {
     const void *x;
     int64_t xsb, xsh, xst;
@@ -383,15 +411,11 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
     float rm = -INFINITY;
     bool rm_nan = false;
     if ((n & (n - 1)) == 0 && n <= 64) {
-        // the n lanes of a token sit side by side inside one wavefront: butterfly over them
-        int bad = is_nan(r) ? 1 : 0;
-        rm = bad ? -INFINITY : r;
-        for (int o = 1; o < n; o <<= 1) {
-            const float other = __shfl_xor(rm, o, 64);
-            bad |= __shfl_xor(bad, o, 64);
-            rm = other > rm ? other : rm;
-        }
-        rm_nan = bad != 0;
+        // the n lanes of a token sit side by side inside one wavefront
+        const int lane = tid & 63;
+        const uint64_t tok_lanes = n == 64 ? ~0ull : ((1ull << n) - 1ull) << (lane / n * n);
+        rm_nan = (__builtin_amdgcn_ballot_w64(is_nan(r)) & tok_lanes) != 0ull;
+        rm = group_max(is_nan(r) ? -INFINITY : r, n, [](float p, float q) { return q > p ? q : p; });
     } else {
         const int base = tok_local * n;
         for (int i = 0; i < n; i++) {
@@ -487,7 +511,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             // the largest finite scale written so far, for the attention kernels' range guard: the wavefront's maximum,
             // and an atomic only when it raises the value (after the first blocks it hardly ever does)
             uint32_t mine = (row_ok && c == 0 && rm < INFINITY) ? __float_as_uint(rm) : 0u;     // scales are positive: bits order like values
-            for (int o = 1; o < 64; o <<= 1) mine = max(mine, (uint32_t)__shfl_xor((int)mine, o, 64));
+            mine = group_max(mine, 64, [](uint32_t p, uint32_t q) { return max(p, q); });
             if ((tid & 63) == 0 && mine > __hip_atomic_load(a.scale_max, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
                 atomicMax(a.scale_max, mine);
         }
