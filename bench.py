@@ -307,7 +307,7 @@ def main():
                      "traffic": RECORDED_TRAFFIC_BYTES.get(T),
                      "traffic_source": f"{TRAFFIC_FILE} (FETCH_SIZE + WRITE_SIZE of an earlier rocprofv3 --pmc run; not "
                                        f"measured by this run)" if T in RECORDED_TRAFFIC_BYTES else None,
-                     "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1>", "kernel_us": round(us_main, 2),
+                     "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1, false>", "kernel_us": round(us_main, 2),
                      "kernel_launch_interval_us": round(us_launch_interval, 2),
                      "algorithmic_bytes_per_launch": cache_bytes,
                      "read_only_kernel_same_grid_us": round(us_read, 2),
