@@ -35,7 +35,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the attention kernel as the FETCH_SIZE / WRITE_SIZE counters read them, recorded offline
 # (rocprofv3 --pmc does not run inside this script); known for these contexts only.
 TRAFFIC_FILE = "profiles/attn_fast_kernel_config2_32k_hbm_traffic.txt"
-RECORDED_TRAFFIC_BYTES = {32768: 37.73e6}
+RECORDED_TRAFFIC_BYTES = {32768: 35.69e6}
 Hq, Hkv, D_H, S, B_R = 32, 8, 128, 96, 4
 
 
