@@ -1024,6 +1024,9 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     if (mb == 16 && p.aux_bits == 3 && CPL == 8 && p.idx_bits == 13 && p.Kc.K <= 4608)
         return two ? launch_one<8, 16, 3, 13, DT, kFastWaves, 2>(p, flags, grid, st, tm) : launch_one<8, 16, 3, 13, DT>(p, flags, grid, st, tm);
     if (mb == 16 && p.aux_bits == 3 && CPL == 8) return launch_one<8, 16, 3, 0, DT>(p, flags, grid, st, tm);
+    // 16 + 1 bits (s192 with four radius bits, the shape of the reference's published prefill figure): generic field decode
+    if (mb == 16 && p.aux_bits == 1 && CPL == 8)
+        return two ? launch_one<8, 16, 1, 0, DT, kFastWaves, 2>(p, flags, grid, st, tm) : launch_one<8, 16, 1, 0, DT>(p, flags, grid, st, tm);
     *handled = false;
     return HQMQ_OK;
 }

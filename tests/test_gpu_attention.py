@@ -87,6 +87,10 @@ CASES = [
     ("fp32 cache", 2, 4, 2, 3, 90, 32, 96, 4, "fp32", False, False, 0, None),
     ("d_h=256", 1, 4, 2, 1, 200, 256, 96, 4, "fp16", False, False, 0, None),
     ("empty and short sequences", 3, 8, 2, 1, 64, 64, 24, 3, "fp16", False, False, 0, [0, 1, 64]),
+    # s192 with four radius bits (the codec of the reference's published prefill figure): 16 + 1 bit layout
+    ("s192_r4 decode, 16+1 bits", 1, 32, 8, 1, 500, 128, 192, 4, "fp16", False, False, 0, None),
+    ("s192_r4 square causal prefill, two column groups", 1, 32, 8, 160, 160, 128, 192, 4, "fp16", False, True, 0, None),
+    ("s192_r4 + Med3x bf16 decode", 2, 8, 4, 1, 333, 128, 192, 4, "bf16", True, False, 0, None),
 ]
 
 
