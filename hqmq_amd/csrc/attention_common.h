@@ -200,13 +200,16 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
     }
 }
 
-// Power-of-two offset of the softmax exponent that keeps P * (V scale) inside fp16: 0 while the largest V scale is
-// below 2^15, else its excess exponent.  Numerator and denominator of the attention output carry the same factor.
+// Power-of-two offset of the softmax exponent that keeps P * (V scale) inside fp16's normal range: 0 while the
+// largest V scale lies in [2^-8, 2^15); above, its excess exponent; below (a cache of tiny values, whose products
+// would be fp16 subnormals), the negative exponent that brings the largest scale to [0.5, 1).  Numerator and
+// denominator of the attention output carry the same factor.
 __device__ __forceinline__ int v_scale_shift_bits(const PackedDev &v) {
     if (!v.scale_max) return 0;
     const uint32_t bits = __builtin_amdgcn_readfirstlane(__builtin_nontemporal_load(v.scale_max));      // wave-uniform
+    if (bits == 0u) return 0;                                   // nothing written yet
     const int e = (int)((bits >> 23) & 0xffu) - 127 + 1;        // scale < 2^e
-    return max(e - 15, 0);
+    return e > 15 ? e - 15 : e < -8 ? e : 0;
 }
 __device__ __forceinline__ float v_scale_shift(const PackedDev &v) { return (float)v_scale_shift_bits(v); }
 

@@ -366,7 +366,7 @@ def attn_fwd(Q: torch.Tensor, Kc, Vc, T_kv: int, *, kv_lens: Optional[torch.Tens
     a.skip_combine = int(skip_combine)
     a.force_generic = int(force_generic)
     a.fp8_table_storage = int(fp8_table_storage)
-    a.wide_range = int(bool(getattr(Vc, "wide_range", False)))      # V scales beyond 2^15: the generic kernel guards the range
+    a.wide_range = int(bool(getattr(Vc, "wide_range", False)))      # V scales outside [2^-8, 2^15): the generic kernel guards the range
     if kernel_events is not None:
         a.start_event, a.stop_event = C.c_void_p(kernel_events[0]), C.c_void_p(kernel_events[1])
     ws = None

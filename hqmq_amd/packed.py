@@ -47,10 +47,11 @@ class PackedTensor:
         # the largest finite scale written so far as fp32 bits (the quantize kernel keeps it up to date): the attention
         # kernels' range guard for bf16 / fp32 caches; fp16 scales cannot leave the range
         self.scale_max = None if dtype == torch.float16 else torch.zeros(1, dtype=torch.int32, device=self.device)
-        # host-side copy of "scale_max has reached 2^15": such a cache takes the layout-generic attention kernel, which
+        # host-side copy of "scale_max lies outside [2^-8, 2^15)": such a cache takes the layout-generic attention kernel, which
         # guards the fp16 range (refresh_range reads the device value; the quantizer calls it after bulk appends and
         # every RANGE_CHECK_EVERY small ones)
         self.wide_range = False
+        self._huge = False
         self._appends_since_range_check = 0
         self.length = 0                      # rows written when all sequences advance together
         self.lengths: Optional[torch.Tensor] = None  # per-sequence rows (int32, device) for ragged batches
@@ -101,17 +102,21 @@ class PackedTensor:
     RANGE_CHECK_EVERY = 256
 
     def refresh_range(self) -> bool:
-        """Reads the largest scale written so far (one device read) and records whether it has reached 2^15, the
-        bound above which the specialised attention kernels would leave the fp16 range.  Only ever switches on."""
-        if self.scale_max is not None and not self.wide_range:
-            self.wide_range = float(self.scale_max.view(torch.float32).item()) >= 32768.0
+        """Reads the largest scale written so far (one device read) and records whether it lies outside [2^-8, 2^15),
+        the range inside which the specialised attention kernels keep P * (V scale) and the verbatim chunks in fp16's
+        normal range.  The largest scale only grows: a cache of tiny values leaves the flag again when larger ones
+        arrive; a cache beyond 2^15 keeps it."""
+        if self.scale_max is not None and not self._huge:
+            v = float(self.scale_max.view(torch.float32).item())
+            self._huge = v >= 32768.0
+            self.wide_range = self._huge or 0.0 < v < 2.0 ** -8
         self._appends_since_range_check = 0
         return self.wide_range
 
     def note_append(self, rows: int) -> None:
         """Called by the quantizer after an append of `rows` rows per sequence: bulk appends (a prefill) and every
         RANGE_CHECK_EVERY-th small one refresh the range flag; never while the stream is being captured."""
-        if self.scale_max is None or self.wide_range:
+        if self.scale_max is None or self._huge:
             return
         self._appends_since_range_check += 1
         if (rows >= 64 or self._appends_since_range_check >= self.RANGE_CHECK_EVERY) and not torch.cuda.is_current_stream_capturing():
@@ -160,6 +165,7 @@ class PackedTensor:
             self._fp8_view = cached
         view = cached[1]
         view.length, view.lengths = self.length, self.lengths
+        view.wide_range, view._huge = self.wide_range, self._huge
         return view
 
     def check_overflow(self) -> None:

@@ -99,8 +99,8 @@ typedef struct hqmq_quantize_args {
     int32_t *stats;           /* [2] or NULL, accumulated: lanes that scored all rows; secondaries kept by the filter */
     uint32_t *scale_max_bits; /* [1] or NULL, accumulated (atomic max): the largest finite per-token scale written to
                                  scale_plane, as the bits of an fp32 number; start it at 0.  The attention kernels read
-                                 it (hqmq_packed.scale_max_bits) to keep caches with scales beyond 2^15 inside the
-                                 fp16 range of their matrix products. */
+                                 it (hqmq_packed.scale_max_bits) to keep caches whose scales lie outside [2^-8, 2^15)
+                                 inside the normal fp16 range of their matrix products. */
 } hqmq_quantize_args;
 int hqmq_quantize(const hqmq_quantize_args *a, void *stream);
 
@@ -185,10 +185,10 @@ typedef struct hqmq_packed {
     int K;                    /* codewords in joint */
     const uint32_t *scale_max_bits; /* [1] or NULL: an upper bound of the finite scales in scale_plane as fp32 bits, as
                                  hqmq_quantize accumulates it.  Read by the layout-generic attention kernel (see
-                                 hqmq_attn_args.wide_range): with a bound of 2^15 or more the softmax weights are carried
-                                 with a power-of-two offset and verbatim outlier chunks are rescaled, so that every
-                                 product stays finite in fp16 (the result is unchanged: numerator and denominator carry
-                                 the same factor).  NULL = all scales are below 2^15 (always true in fp16). */
+                                 hqmq_attn_args.wide_range): with a bound of 2^15 or more, or below 2^-8, the softmax
+                                 weights are carried with a power-of-two offset and verbatim outlier chunks are rescaled,
+                                 so that every product stays finite and normal in fp16 (the result is unchanged: numerator
+                                 and denominator carry the same factor).  NULL = no offset. */
 } hqmq_packed;
 
 /* Dense decode of a packed cache (outlier chunks substituted from the sideband).
@@ -232,11 +232,12 @@ typedef struct hqmq_attn_args {
                                  gather as :133-135 there does).  Same results as 0 on such tables; honoured by the
                                  specialised decode kernels of the 16-bit layouts at d_h 128, ignored elsewhere. */
     int wide_range;           /* 1: a bf16 cache whose per-token scales may reach 2^15 (or whose verbatim outlier values may
-                                 exceed 65504).  The specialised kernels multiply the softmax weights with the V scales in
-                                 fp16 and would overflow; such a cache takes the layout-generic kernel, which reads
-                                 hqmq_packed.scale_max_bits and keeps every product inside the fp16 range (fp32 caches always
-                                 take it).  Callers that track the bound (hqmq_quantize_args.scale_max_bits) set this when it
-                                 reaches 2^15; data of ordinary magnitude never does. */
+                                 exceed 65504), or whose largest scale is below 2^-8.  The specialised kernels multiply the
+                                 softmax weights with the V scales in fp16 and would overflow, or lose the product to fp16
+                                 subnormals; such a cache takes the layout-generic kernel, which reads
+                                 hqmq_packed.scale_max_bits and keeps every product inside the normal fp16 range (fp32 caches
+                                 always take it).  Callers that track the bound (hqmq_quantize_args.scale_max_bits) set this
+                                 when it leaves [2^-8, 2^15); data of ordinary magnitude never does. */
 } hqmq_attn_args;
 int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, int n_splits);
 /* The n_splits hqmq_attn_fwd would choose; ragged = 1 when kv_len is passed (more, smaller blocks). */
