@@ -273,3 +273,39 @@ def test_ragged_append_with_positions():
         untouched = torch.ones(64, dtype=torch.bool)
         untouched[p:p + 2] = False
         assert int(cache.K.main[b][:, untouched].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("S,b_r", [(24, 3), (24, 4), (7, 2), (96, 4), (96, 3), (96, 6), (192, 6), (192, 4), (300, 5)])
+@pytest.mark.parametrize("d_h", [16, 20, 80, 128, 160, 256])
+def test_packed_planes_of_every_layout_and_head_size(S, b_r, d_h):
+    """The planes a quantize call packs, read back by the independent bit reader of tests/helpers.py, hold the codes,
+    flags and scales the same call returns: every width the layout rule produces (8 / 12 / 16 bits in the main plane,
+    0 - 4 in the aux plane), head sizes whose lanes do and do not sit side by side in a wavefront (n = 4 ... 64, with
+    20 and 40 not powers of two), one-token, short and bulk calls, with and without Med3x, and the filter search
+    against the exhaustive scan (algo = 1) on the same input."""
+    from hqmq_amd.packed import PackedTensor
+    from tests.helpers import unpack_planes
+    ops = _ops()
+    g = torch.Generator().manual_seed(1000 * S + 10 * d_h + b_r)
+    H, n = 2, d_h // 4
+    for dn in ("fp16", "bf16"):
+        dt = DT[dn]
+        J, slack = ops.build_joint(torch.randn(H, S, 4, generator=g).to(DEV), dt)
+        for B, T, outl in ((2, 1, True), (1, 5, False), (2, 70, True)):
+            if outl and n > 32:
+                continue                                                     # the sideband takes at most 32 chunks per token
+            spread = torch.exp(torch.randn(B, H, T, n, 1, generator=g)).expand(B, H, T, n, 4).reshape(B, H, T, d_h)
+            x = (torch.randn(B, H, T, d_h, generator=g) * spread).to(dt).to(DEV)
+            pt = PackedTensor(B, H, T, d_h, S, b_r, dt, DEV, joint=J, outliers=outl)
+            thr = ops.med3x_threshold(x, 3.0)[1] if outl else None
+            r = ops.quantize(x, J, slack, b_r, want_codes=True, thr=thr, want_mask=outl, cache=pt, t_off=0)
+            scan = ops.quantize(x, J, slack, b_r, want_codes=True, algo=1)
+            assert torch.equal(r["idx"], scan["idx"]) and torch.equal(r["rq"], scan["rq"]), (dn, B, T)
+            for b in range(B):
+                idx, rq, flags = unpack_planes(pt, b, T)
+                want_rq = r["rq"][b].long()
+                if outl:
+                    assert torch.equal(flags, r["mask"][b].bool()), (dn, B, T, "flags")
+                    want_rq = torch.where(r["mask"][b].bool(), torch.zeros_like(want_rq), want_rq)   # flagged: radius code 0
+                assert torch.equal(idx, r["idx"][b].long()) and torch.equal(rq, want_rq), (dn, B, T, "codes")
+                assert bit_equal(pt.scale[b, :, :T], r["r_max"][b]), (dn, B, T, "scales")
