@@ -434,7 +434,8 @@ extern "C" int64_t hqmq_attn_workspace_bytes(int B, int H_q, int T_q, int d_h, i
 }
 
 // Blocks per (sequence, KV head, column group): one block per CU, each of a block's eight wavefronts
-// keeping at least one 64-token super-tile.
+// keeping at least one 32-token half-step (short contexts are bound by the launch's fixed costs: at 4k and 8k
+// tokens twice the blocks of half the length measure 9 % faster).
 extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv, int ragged) {
     if (B < 1 || H_q < 1 || H_kv < 1 || T_q < 1 || T_kv < 1) return 1;
     const int G = H_q / H_kv;
@@ -442,7 +443,7 @@ extern "C" int hqmq_attn_pick_splits(int B, int H_q, int H_kv, int T_q, int T_kv
     // sequences of different lengths: four rounds of smaller blocks even out the finishing times
     const int64_t target = ragged ? 1024 : 256;
     int64_t s = (target + base - 1) / base;
-    const int64_t cap = (T_kv + 8 * kSuper - 1) / (8 * kSuper);
+    const int64_t cap = (T_kv + 4 * kSuper - 1) / (4 * kSuper);
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     if (s > 512) s = 512;

@@ -390,7 +390,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
     int per_wave = (b_end - b_begin + WV - 1) / WV;
-    constexpr int kWaveStep = WV == 12 ? 32 : kSuper;        // ranges of whole half-steps; 64 keeps the 8-wave split as tuned
+    constexpr int kWaveStep = 32;        // ranges of whole half-steps
     per_wave = (per_wave + kWaveStep - 1) / kWaveStep * kWaveStep;
     // every super-tile starts at a multiple of 64 below T_kv <= t_cap (a multiple of 64): whole tiles are readable
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);

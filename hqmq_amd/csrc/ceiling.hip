@@ -27,7 +27,7 @@ __global__ __launch_bounds__(WV * 64) void read_ceiling_kernel(const uint8_t *km
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(sp * per_split, Tkv), b_end = min(Tkv, b_begin + per_split);
     int per_wave = (b_end - b_begin + WV - 1) / WV;
-    constexpr int kWaveStep = WV == 12 ? 32 : kSuper;
+    constexpr int kWaveStep = 32;
     per_wave = (per_wave + kWaveStep - 1) / kWaveStep * kWaveStep;
     const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
     constexpr int mrb = 64;
