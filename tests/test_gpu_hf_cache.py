@@ -66,6 +66,57 @@ def test_packed_cache_matches_fake_quant_cache(dn, med3x):
     assert packed.nbytes() < (0.6 if med3x else 0.36) * dense_bytes
 
 
+@pytest.mark.parametrize("med3x", [False, True])
+@pytest.mark.parametrize("dn", ["fp16", "bf16"])
+def test_attention_inside_the_model_meets_the_kernel_bound(dn, med3x, monkeypatch):
+    """Parity of the attention calls the model itself makes: every decode-step call of the fused kernel inside the HF
+    forward pass (real activations: RoPE'd queries, the layers' own K / V with planted outlier channels) is checked
+    against two fp32 references computed from the codes in that layer's packed cache, with the bound the kernel is
+    held to everywhere else (tests/helpers.py:assert_attention_close)."""
+    import hqmq
+    import hqmq_amd.hf_cache as hf
+    from hqmq_amd import ops
+    from src.model_utils import ATTN_NAME, PackedQuantizedCache
+    from tests.helpers import assert_attention_close, exact_dense, gpu_attention_refs
+    dt = {"fp16": torch.float16, "bf16": torch.bfloat16}[dn]
+    model = tiny_llama(dt)
+    q = hqmq.HQMQ(n_layers=3, n_heads=2, secondary_size=96, radius_bits=4, device=DEV)
+    if med3x:
+        q = hqmq.with_outlier_extraction(q, C=3.0)
+        with torch.no_grad():
+            for layer in model.model.layers:
+                layer.self_attn.k_proj.weight[8:16] *= 12.0
+                layer.self_attn.v_proj.weight[40:44] *= 12.0
+    calls = []
+    inner = hf.fused_attention_packed
+
+    def recording(query, cache, **kw):
+        out = inner(query, cache, **kw)
+        if query.shape[2] == 1:
+            calls.append((query.clone(), cache, kw["T_kv"], out.clone()))
+        return out
+    monkeypatch.setattr(hf, "fused_attention_packed", recording)
+    ids = torch.randint(0, 256, (2, 150), generator=torch.Generator().manual_seed(5)).to(DEV)
+    model.set_attn_implementation(ATTN_NAME)
+    cache = PackedQuantizedCache(q, max_tokens=256, sideband_frac=0.5)
+    with torch.no_grad():
+        model(ids[:, :147], past_key_values=cache, use_cache=True)
+        for t in range(147, 150):
+            model(ids[:, t:t + 1], past_key_values=cache, use_cache=True)
+    cache.check_overflow()
+    assert len(calls) == 9                                      # three layers, three decode steps
+    worst = 0.0
+    for query, packed, L, out in calls:
+        K_D, V_D = ops.dequant_packed(packed.K, L, 0), ops.dequant_packed(packed.V, L, 0)
+        for b in range(query.shape[0]):
+            # flagged chunks are verbatim in the dense decode: it serves as the source of their exact values
+            K_x, V_x = exact_dense(packed.K, b, L, K_D[b]), exact_dense(packed.V, b, L, V_D[b])
+            ref_d, ref_x, a_abs = gpu_attention_refs(query[b, :, 0], K_D[b].float(), V_D[b].float(), K_x, V_x)
+            worst = max(worst, assert_attention_close(out[b, :, 0], ref_d.cpu(), ref_x.cpu(), a_abs.cpu(), base=2e-3,
+                                                      what=f"{dn} med3x={med3x} L={L} sequence {b}"))
+    print(f"\n{dn} med3x={med3x}: attention calls inside the model, max |O - ref_D| {worst:.3e}")
+
+
 def test_packed_cache_crop_replays_identically():
     """Rolling the packed cache back (speculative decoding) and decoding the same tokens again gives the same logits
     bit for bit, with outliers on both sides of the cut."""
