@@ -91,6 +91,13 @@ CASES = [
     ("s192_r4 decode, 16+1 bits", 1, 32, 8, 1, 500, 128, 192, 4, "fp16", False, False, 0, None),
     ("s192_r4 square causal prefill, two column groups", 1, 32, 8, 160, 160, 128, 192, 4, "fp16", False, True, 0, None),
     ("s192_r4 + Med3x bf16 decode", 2, 8, 4, 1, 333, 128, 192, 4, "bf16", True, False, 0, None),
+    # the other widths of the layout rule at d_h 128
+    ("s96_r6 decode, 16+2 bits", 1, 32, 8, 1, 500, 128, 96, 6, "fp16", False, False, 0, None),
+    ("s192_r5 + Med3x prefill chunk, 16+2 bits", 1, 8, 2, 40, 300, 128, 192, 5, "bf16", True, True, 260, None),
+    ("s24_r4 decode ragged, 12+2 bits", 3, 8, 4, 1, 400, 128, 24, 4, "bf16", False, False, 0, [400, 77, 256]),
+    ("s24_r4 + Med3x decode, 12+2 bits", 2, 8, 4, 1, 200, 128, 24, 4, "fp16", True, False, 0, None),
+    ("s96_r3 decode, 12+3 bits", 1, 32, 8, 1, 500, 128, 96, 3, "fp16", False, False, 0, None),
+    ("s24_r5 square causal prefill, 12+3 bits, two column groups", 1, 32, 8, 160, 160, 128, 24, 5, "fp16", False, True, 0, None),
 ]
 
 
