@@ -214,7 +214,7 @@ __device__ __forceinline__ int v_scale_shift_bits(const PackedDev &v) {
 __device__ __forceinline__ float v_scale_shift(const PackedDev &v) { return (float)v_scale_shift_bits(v); }
 
 // Implemented in attention_fast.hip: kernels specialised at compile time for the common layouts
-// (d_h 64/128, fp16/bf16 caches, 16+0 / 12+1 / 16+3 bit codes). Returns HQMQ_OK and sets *handled when
+// (d_h 64/128, fp16/bf16 caches; 16+0 / 12+1 / 16+3 bit codes, and at d_h 128 the widths 16+1, 16+2, 12+2, 12+3). Returns HQMQ_OK and sets *handled when
 // it launched one of them; otherwise the caller falls back to the generic kernel.
 // Optional events that receive the GPU timestamps of the begin and the end of the main attention kernel.
 struct LaunchTiming {
