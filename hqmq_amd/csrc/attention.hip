@@ -533,6 +533,14 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
             p.scale_vec = 0;
     if (p.n_cg > 65535) return HQMQ_ERR_SHAPE;
     dim3 grid((unsigned)n_splits, (unsigned)p.n_cg, (unsigned)(a->B * a->H_kv));
+    {
+        const uint64_t gx = grid.x, gy = grid.y, gz = grid.z;
+        p.m_gz = attn_div_magic(gz, gx * gy * gz);
+        p.m_gx = attn_div_magic(gx, gx * gy);
+        p.m_hkv = attn_div_magic((uint64_t)a->H_kv, gz);
+        p.m_G = attn_div_magic((uint64_t)p.G, gy * 16);
+        p.m_splits = attn_div_magic((uint64_t)n_splits, (uint64_t)a->T_kv + (uint64_t)n_splits);
+    }
     hipStream_t st = (hipStream_t)stream;
     LaunchTiming tm;
     tm.start = (hipEvent_t)a->start_event;

@@ -48,6 +48,8 @@ struct AttnParams {
     int scale_vec;  // scales of 4 consecutive tokens may be read with one aligned vector load
     float *ws;      // split partials [row][split][kPartialHead + d_h]: m (base-2 exponent units), l, two unused floats, acc
     int xcd_remap;  // blocks of one (sequence, KV head) share an XCD (see attn_fast_kernel)
+    // multipliers that replace the index divisions of the kernels' prologue (attn_div_magic; 0 = divide)
+    unsigned m_hkv, m_G, m_gz, m_gx, m_splits;
     int tab_fp8;    // both tables hold e4m3 numbers and the caller asks for float8 storage in LDS
     int wide_range; // scales or verbatim values of the cache may leave the fp16 range: layout-generic kernel only
 };
@@ -198,6 +200,12 @@ __device__ __forceinline__ void fill_table(uint2 *dst, const void *joint, int dt
             if (k < K) dst[k] = __builtin_bit_cast(uint2, tmp[u]);
         }
     }
+}
+
+// ceil(2^32 / d) if x / d == umulhi(x, that) for every x <= x_max (true while x_max * d < 2^32), else 0
+inline unsigned attn_div_magic(uint64_t d, uint64_t x_max) {
+    if (d < 2 || x_max * d >= (1ull << 32)) return 0u;
+    return (unsigned)(((1ull << 32) + d - 1) / d);
 }
 
 // Power-of-two offset of the softmax exponent that keeps P * (V scale) inside fp16's normal range: 0 while the

@@ -287,6 +287,10 @@ __device__ __forceinline__ void scale_chunks(const half4 (&g)[CPL], const half2v
     for (int j = 0; j < CPL; j++) a[j] = PS ? g[j] : g[j] * r[j >> 1][j & 1];
 }
 
+// x / d through the multiplier the host worked out for d (m = ceil(2^32 / d), exact while x * d < 2^32; 0 where that
+// cannot be promised or d = 1: then the division itself)
+__device__ __forceinline__ unsigned fast_div(unsigned x, unsigned d, unsigned m) { return m ? __umulhi(x, m) : d == 1u ? x : x / d; }
+
 __device__ __forceinline__ half8 cat8(half4 x, half4 y) { return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7); }
 
 // max over the four 16-lane rows (lanes l, l^16, l^32, l^48) without going through LDS
@@ -342,12 +346,26 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         // the hardware hands workgroups to the XCDs round-robin in linear order (x fastest): renumber so that the
         // (sequence, KV head) index runs fastest and, with a multiple of eight of them, stays on one XCD
         const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-        const unsigned r = lin / gridDim.z;
+        const unsigned r = fast_div(lin, gridDim.z, p.m_gz);
         bz = (int)(lin - r * gridDim.z);
-        by = (int)(r / gridDim.x);
+        by = (int)fast_div(r, gridDim.x, p.m_gx);
         bx = (int)(r - (unsigned)by * gridDim.x);
     }
-    const int slot = bz / p.Hkv, hkv = bz - slot * p.Hkv;
+    const int slot = (int)fast_div((unsigned)bz, (unsigned)p.Hkv, p.m_hkv), hkv = bz - slot * p.Hkv;
+    // The codeword-table loads are the longest dependency chain of the prologue (load, convert, LDS store, barrier)
+    // and need nothing but the KV head: they are requested before anything else is worked out.  16-byte loads of two
+    // codewords, all unconditional (clamped): straight-line code, exact wait counts.
+    constexpr int FU = 3;
+    const uint4v *ksrc = (const uint4v *)((const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4));
+    const uint4v *vsrc = (const uint4v *)((const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4));
+    const int Kk2 = p.Kc.K >> 1, Kv2 = p.Vc.K >> 1;        // tables of an even number of codewords (checked at launch)
+    uint4v tk[FU], tv[FU];
+#pragma unroll
+    for (int u = 0; u < FU; u++) {
+        const int k = threadIdx.x + u * NT;
+        tk[u] = ksrc[min(k, Kk2 - 1)];
+        tv[u] = vsrc[min(k, Kv2 - 1)];
+    }
     const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
     const int bh = b * p.Hkv + hkv;
     const int cg0 = by * NCG, sp = bx;
@@ -364,7 +382,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     for (int cgi = 0; cgi < NCG; cgi++) {
         const int cidx = (cg0 + cgi) * 16 + col;
         col_ok[cgi] = cidx < p.Tq * G;
-        tq[cgi] = col_ok[cgi] ? cidx / G : 0;
+        tq[cgi] = col_ok[cgi] ? (int)fast_div((unsigned)cidx, (unsigned)G, p.m_G) : 0;
         hq[cgi] = hkv * G + (col_ok[cgi] ? cidx - tq[cgi] * G : 0);
         int64_t lim64 = kv_end;
         if (p.causal) lim64 = min(lim64, (int64_t)tq[cgi] + p.causal_offset + 1);
@@ -386,7 +404,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // tokens before kv_start[b] are invisible (left padding): the walk starts at the super-tile that holds it
     const int col_start = p.kv_start ? min(max(p.kv_start[b], 0), blk_lim) : 0;
     const int blk_lo = col_start / kSuper * kSuper;
-    int per_split = (blk_lim - blk_lo + p.n_splits - 1) / p.n_splits;
+    int per_split = (int)fast_div((unsigned)(blk_lim - blk_lo + p.n_splits - 1), (unsigned)p.n_splits, p.m_splits);
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
     int per_wave = (b_end - b_begin + WV - 1) / WV;
@@ -488,22 +506,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     };
 
-    // First batch of codeword-table loads (the longest dependency chain of the prologue: load, convert, LDS
-    // store, barrier), then the wavefront's first super-tile; the LDS stores follow.  The Q rows were requested
-    // before both so that waiting for them does not wait for the tiles.
-    // 16-byte loads of two codewords, all unconditional (clamped): straight-line code, exact wait counts
-    constexpr int FU = 3;
-    const uint4v *ksrc = (const uint4v *)((const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4));
-    const uint4v *vsrc = (const uint4v *)((const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4));
-    const int Kk2 = p.Kc.K >> 1, Kv2 = p.Vc.K >> 1;        // tables of an even number of codewords (checked at launch)
-    uint4v tk[FU], tv[FU];
-#pragma unroll
-    for (int u = 0; u < FU; u++) {
-        const int k = threadIdx.x + u * NT;
-        tk[u] = ksrc[min(k, Kk2 - 1)];
-        tv[u] = vsrc[min(k, Kv2 - 1)];
-    }
-
     FastTile<NW, AB, FLAGS, NH> cur;
     FlagTile f0 = {}, f1 = {};
     {
@@ -514,6 +516,11 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         load_super(t_first, cur);
         if (FLAGS) load_flags(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);        // made ready below
     }
+    // Plain variants keep two half-steps in flight; the second is requested right behind the first (both queue
+    // behind the table loads, which were requested at the very start).
+    auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
+    FastTile<NW, AB, FLAGS, NH> tb;
+    if constexpr (!FLAGS) load_super(readable(t_begin + 32 < t_end ? t_begin + 32 : t_begin), tb);
 
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
@@ -549,14 +556,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             }
             if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT, F8>(ktab, ksrc, Kk2, vtab, vsrc, Kv2, FU * NT);
         }
-    }
-    // Plain variants keep two half-steps in flight.  The second one is requested only now, when the table loads
-    // have come back: requested at the start it would queue in front of them and delay the whole block.
-    auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
-    FastTile<NW, AB, FLAGS, NH> tb;
-    if constexpr (!FLAGS) {
-        asm volatile("" ::: "memory");
-        load_super(readable(t_begin + 32 < t_end ? t_begin + 32 : t_begin), tb);
     }
     if (FLAGS && threadIdx.x >= 64 && threadIdx.x < 100) {
         const uint32_t w = threadIdx.x - 64, row = w >> 2, d = w & 3;
