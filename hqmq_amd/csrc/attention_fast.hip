@@ -332,7 +332,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     constexpr int NT = WV * 64;
     constexpr int kKPre = CPL >= 8 ? 3 : 1;     // batches of outlier entries requested ahead (d_h 64 has half the chunks)
     constexpr bool kBatchGathers = false;       // see half_step: measured, no gain on any shape (178 against 157 registers)
-    constexpr int NH = 1, STEP = 32 * NH;       // prefetch distance in half-steps: one measures faster than two on every shape
+    constexpr int NH = 1;       // half-steps per prefetched tile: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
     constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
     constexpr int VTAB = vtab_offset(PS), QOFF = q_offset(PS), SELOFF = sel_offset(PS);
@@ -407,12 +407,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     int per_split = (int)fast_div((unsigned)(blk_lim - blk_lo + p.n_splits - 1), (unsigned)p.n_splits, p.m_splits);
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
-    int per_wave = (b_end - b_begin + WV - 1) / WV;
-    constexpr int kWaveStep = 32;        // ranges of whole half-steps
-    per_wave = (per_wave + kWaveStep - 1) / kWaveStep * kWaveStep;
-    // every super-tile starts at a multiple of 64 below T_kv <= t_cap (a multiple of 64): whole tiles are readable
-    const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
-
+    // The block's half-steps go to its wavefronts round-robin: wavefront w takes the 32 tokens at b_begin + 32 (w + i WV),
+    // i = 0, 1, ...  What the wavefronts of a block request at any one time is then one contiguous stretch of the
+    // planes (batch 8: 3.5 % faster than a contiguous range per wavefront, ragged config 4: 2 %).
+    // Every half-step starts at a multiple of 32 below T_kv <= t_cap (a multiple of 64): whole tiles are readable.
+    constexpr int TS = 32 * WV;
+    const int t_begin = min(b_begin + wave * 32, b_end), t_end = b_end;
     const size_t plane_row0 = (size_t)bh * p.t_cap;
     constexpr int mrb = n * MB / 8, arb = (n * AB + 7) / 8;
     const int64_t tiles_cap = p.t_cap / kTile;
@@ -514,13 +514,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const int t_first = min(t_begin, (int)p.t_cap - 32);
         if (FLAGS) load_flags(t_first, f0);
         load_super(t_first, cur);
-        if (FLAGS) load_flags(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);        // made ready below
+        if (FLAGS) load_flags(t_begin + TS < t_end ? t_begin + TS : t_first, f1);        // made ready below
     }
     // Plain variants keep two half-steps in flight; the second is requested right behind the first (both queue
     // behind the table loads, which were requested at the very start).
     auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
     FastTile<NW, AB, FLAGS, NH> tb;
-    if constexpr (!FLAGS) load_super(readable(t_begin + 32 < t_end ? t_begin + 32 : t_begin), tb);
+    if constexpr (!FLAGS) load_super(readable(t_begin + TS < t_end ? t_begin + TS : t_begin), tb);
 
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
@@ -869,7 +869,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     if constexpr (FLAGS) {
         const int t_first = min(t_begin, (int)p.t_cap - 32);
         flags_ready(t_first, f0);
-        flags_ready(t_begin + STEP < t_end ? t_begin + STEP : t_first, f1);
+        flags_ready(t_begin + TS < t_end ? t_begin + TS : t_first, f1);
         if (t_begin < t_end) issue_all(f0, kc, vc);
     }
 
@@ -879,35 +879,35 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         int t0 = t_begin;
         if (t0 < t_end) {
             while (true) {
-                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), tc);
+                load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), tc);
                 half_step(cur.h[0], t0, kc, vc);
-                t0 += 32;
+                t0 += TS;
                 if (t0 >= t_end) break;
-                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), cur);
+                load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), cur);
                 half_step(tb.h[0], t0, kc, vc);
-                t0 += 32;
+                t0 += TS;
                 if (t0 >= t_end) break;
-                load_super(readable(t0 + 64 < t_end ? t0 + 64 : t0), tb);
+                load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), tb);
                 half_step(tc.h[0], t0, kc, vc);
-                t0 += 32;
+                t0 += TS;
                 if (t0 >= t_end) break;
             }
         }
     }
-    for (int t0 = t_begin; FLAGS && t0 < t_end; t0 += STEP) {
+    for (int t0 = t_begin; FLAGS && t0 < t_end; t0 += TS) {
         FastTile<NW, AB, FLAGS, NH> nxt;
         FlagTile f2 = {};
         KPre<kKPre> kn = {};
         VPre<kVPre> vn = {};
-        const bool more = t0 + STEP < t_end, more2 = t0 + 2 * STEP < t_end;
+        const bool more = t0 + TS < t_end, more2 = t0 + 2 * TS < t_end;
         if (FLAGS) {
             // tile offsets two steps ahead, sideband entries one step ahead (their offsets were requested a step
             // ago); past the end the current tile is requested again
-            load_super(more ? t0 + STEP : t0, nxt);
-            load_flags(more2 ? t0 + 2 * STEP : t0, f2);           // made ready at the end of this half-step
+            load_super(more ? t0 + TS : t0, nxt);
+            load_flags(more2 ? t0 + 2 * TS : t0, f2);           // made ready at the end of this half-step
             issue_all(f1, kn, vn);
         } else if (more) {
-            load_super(t0 + STEP, nxt);
+            load_super(t0 + TS, nxt);
         }
         half_step(cur.h[0], t0, kc, vc);
         if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, kc, vc);
@@ -916,7 +916,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             if (FLAGS) {
                 kc = kn;
                 vc = vn;
-                flags_ready(more2 ? t0 + 2 * STEP : t0, f2);
+                flags_ready(more2 ? t0 + 2 * TS : t0, f2);
                 f1 = f2;
             }
         }

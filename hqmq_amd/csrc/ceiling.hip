@@ -1,5 +1,5 @@
 // Measurement aid: a kernel that only READS the planes of a packed cache, with the grid, the per-wavefront token
-// ranges and the per-lane load pattern of the specialised decode-attention kernel (16-byte loads of the main
+// half-steps and the per-lane load pattern of the specialised decode-attention kernel (16-byte loads of the main
 // rows of K and V, 8-byte loads of four scales, 32 tokens per step), and a ring of DEPTH such steps in flight.
 // Its duration is what the memory system allows a kernel of this shape; the attention kernel's distance from it
 // is what its own arithmetic, tables and merge cost.  Supports the 16+0 layout at d_h = 128 (s96_r4), no sideband.
@@ -26,10 +26,9 @@ __global__ __launch_bounds__(WV * 64) void read_ceiling_kernel(const uint8_t *km
     int per_split = (Tkv + n_splits - 1) / n_splits;
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
     const int b_begin = min(sp * per_split, Tkv), b_end = min(Tkv, b_begin + per_split);
-    int per_wave = (b_end - b_begin + WV - 1) / WV;
-    constexpr int kWaveStep = 32;
-    per_wave = (per_wave + kWaveStep - 1) / kWaveStep * kWaveStep;
-    const int t_begin = min(b_begin + wave * per_wave, b_end), t_end = min(b_end, t_begin + per_wave);
+    // half-steps round-robin over the block's wavefronts, as in the attention kernel
+    constexpr int STRIDE = 32 * WV;
+    const int t_begin = min(b_begin + wave * 32, b_end), t_end = b_end;
     constexpr int mrb = 64;
     const uint8_t *k_rows = kmain + (size_t)bh * t_cap * mrb + col * mrb + grp * 16;
     const uint8_t *v_rows = vmain + (size_t)bh * t_cap * mrb + col * mrb + grp * 16;
@@ -57,16 +56,16 @@ __global__ __launch_bounds__(WV * 64) void read_ceiling_kernel(const uint8_t *km
     StepWords ring[DEPTH];
     if (t_begin < t_end) {
 #pragma unroll
-        for (int d = 0; d < DEPTH - 1; d++) load(t_begin + 32 * d < t_end ? t_begin + 32 * d : t_begin, ring[d]);
+        for (int d = 0; d < DEPTH - 1; d++) load(t_begin + STRIDE * d < t_end ? t_begin + STRIDE * d : t_begin, ring[d]);
         int t = t_begin;
         while (true) {
             bool done = false;
 #pragma unroll
             for (int d = 0; d < DEPTH; d++) {
-                const int tn = t + 32 * (DEPTH - 1);
+                const int tn = t + STRIDE * (DEPTH - 1);
                 load(tn < t_end ? tn : t, ring[(d + DEPTH - 1) % DEPTH]);
                 consume(ring[d]);
-                t += 32;
+                t += STRIDE;
                 if (t >= t_end) { done = true; break; }
             }
             if (done) break;
