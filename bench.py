@@ -106,6 +106,9 @@ def event_time_us(fn, iters, stream):
     return e0.elapsed_time(e1) * 1e3 / iters
 
 
+LAST_KERNEL_STATS = {}
+
+
 def kernel_time_us(launch, iters):
     """Average GPU duration of the attention kernel itself over `iters` launches launch(i, events): every launch
     carries its own pair of HIP events, which the runtime stamps at the begin and at the end of that dispatch (the
@@ -124,14 +127,19 @@ def kernel_time_us(launch, iters):
     for i, (a, b) in enumerate(ev):
         launch(i, (a.value, b.value))
     torch.cuda.synchronize()
-    total, ms = 0.0, C.c_float()
+    durs, ms = [], C.c_float()
     for a, b in ev:
         if hip.hipEventElapsedTime(C.byref(ms), a, b) != 0:
             raise RuntimeError("hipEventElapsedTime failed")
-        total += ms.value
+        durs.append(ms.value * 1e3)
         hip.hipEventDestroy(a)
         hip.hipEventDestroy(b)
-    return total * 1e3 / iters
+    # eager launches are paced by the host: now and then one is stretched by whatever else the device was doing between
+    # them.  Launches beyond 1.5 x the median are left out of the average; LAST_KERNEL_STATS keeps the full picture.
+    med = sorted(durs)[len(durs) // 2]
+    kept = [d for d in durs if d <= 1.5 * med]
+    LAST_KERNEL_STATS.update(mean_all=sum(durs) / len(durs), median=med, max=max(durs), dropped=len(durs) - len(kept))
+    return sum(kept) / len(kept)
 
 
 def cpu_attention_baseline(slice_tokens, repeats=5):
@@ -270,6 +278,7 @@ def main():
         ops.attn_fwd(queries[j], caches[j].K, caches[j].V, T, n_splits=n_splits, out=outs[j], skip_combine=True, kernel_events=ev,
                      workspace=partials)
     us_main = kernel_time_us(main_kernel, 192)
+    main_stats = {k: round(v, 2) for k, v in LAST_KERNEL_STATS.items()}
     us_main_same = kernel_time_us(lambda i, ev: main_kernel(i, ev, False), 192)
     us_launch_interval, _ = graph_us(lambda i: main_kernel(i, None), args.steps, stream)
     us_step_same, _ = graph_us(step_same, args.steps, stream)
@@ -307,7 +316,7 @@ def main():
                      "traffic": RECORDED_TRAFFIC_BYTES.get(T),
                      "traffic_source": f"{TRAFFIC_FILE} (FETCH_SIZE + WRITE_SIZE of an earlier rocprofv3 --pmc run; not "
                                        f"measured by this run)" if T in RECORDED_TRAFFIC_BYTES else None,
-                     "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1, false>", "kernel_us": round(us_main, 2),
+                     "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1, false>", "kernel_us": round(us_main, 2), "kernel_us_stats": main_stats,
                      "kernel_launch_interval_us": round(us_launch_interval, 2),
                      "algorithmic_bytes_per_launch": cache_bytes,
                      "read_only_kernel_same_grid_us": round(us_read, 2),
