@@ -275,7 +275,8 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                     float b2 = best2_mfma(vv[0], vv[1], vv[2], vv[3]);
                     if (decltype(tail)::value && sn - slots >= S) b2 = -INFINITY;      // behind the slot's last secondary
                     b2v[i] = b2;
-                    asm("v_max_f32_e32 %0, %1, %2" : "=v"(m2) : "v"(m2), "v"(b2));      // both are ordinary numbers here
+                    // the running maximum takes two scores at a time (all ordinary numbers or -inf here)
+                    if (i & 1) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(m2) : "v"(m2), "v"(b2v[i - 1]), "v"(b2));
                 }
                 const float thr = m2 - margin2;
                 uint32_t word = 0u;
