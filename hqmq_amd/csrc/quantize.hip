@@ -115,6 +115,26 @@ __device__ __forceinline__ float best2_mfma(float v0, float v1, float v2, float 
     return fmaxf(mx + mx, sum);
 }
 
+// What the doubled filter score of a secondary must reach for one of its codewords to be able to win, given the
+// largest doubled filter score m2 seen so far.  The reference rounds every score once to D.  The unrounded
+// reference score of the best codeword is at least x = m2 / 2 less the errors of the filter and of the table, so
+// the winning rounded score is at least R = RNE_D(x), and only unrounded scores from the midpoint below R upwards
+// round that high.  Taking the table and filter errors off once more turns that midpoint into a bound on the
+// filter score.  On average this is half a unit in the last place of D tighter than the worst-case margin, which
+// it never undercuts (the larger of the two bounds is returned; both hold).
+template <class D>
+__device__ __forceinline__ float candidate_threshold(float m2, float table_err, float filter_err, float margin2) {
+    const float worst = m2 - margin2;
+    if (D::code == HQMQ_F32) return worst;
+    const float x = 0.5f * (m2 - 0.5f * filter_err) - table_err;
+    const float R = D::rnd(x);
+    // R is a normal number of D here, so the number of D below it is one step of D's last mantissa bit down
+    const float below = __uint_as_float(__float_as_uint(R) - (D::code == HQMQ_F16 ? 1u << 13 : 1u << 16));
+    const float mid = 0.5f * (R + below);
+    const float thr = 2.f * (mid - table_err) - 0.5f * filter_err;
+    return R > 1.0e-4f ? fmaxf(thr, worst) : worst;
+}
+
 // twice the exact score of Hurwitz unit p for rotated chunk v
 __device__ __forceinline__ float exact2_of(const float v[4], int p) {
     if (p < 8) {
@@ -245,8 +265,10 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
         float us[4];
         for (int j = 0; j < 4; j++) us[j] = search ? u[j] : (j == 0 ? 1.f : 0.f);
         const float ulen = sqrtf(fmaf(us[3], us[3], fmaf(us[2], us[2], fmaf(us[1], us[1], us[0] * us[0])))) * 1.000001f;
-        const float E = ulen * (a.slack[h] + 1.01f * D::eps() + 9.5367e-7f);
-        const float margin2 = 4.f * E + ulen * 7.6294e-6f + 1.0e-6f;
+        const float table_err = ulen * (a.slack[h] + 9.5367e-7f);      // unrounded reference score vs exact score
+        const float filter_err = ulen * 7.6294e-6f + 1.0e-6f;           // doubled filter score vs twice the exact score
+        const float E = table_err + ulen * 1.01f * D::eps();
+        const float margin2 = 4.f * E + filter_err;
         float m2 = -INFINITY;
         int cnt = 0;
         if (D::code != HQMQ_F32) {
@@ -256,12 +278,13 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
             const half4 ub = half4{(_Float16)us[0], (_Float16)us[1], (_Float16)us[2], (_Float16)us[3]};
             const uint2 *acol = rot + (tid & 3);
             // The scan runs in blocks of 32 secondaries whose scores stay in registers.  Only the running maximum is
-            // kept inside a block; at its end the secondaries within the margin of the maximum so far become a bit mask
-            // (a compare and an add-with-carry each) and go into the list of the re-score below.  A maximum that has
-            // moved up by more than the margin during the block leaves everything listed before more than the margin
-            // below the final maximum: the list starts over.
+            // kept inside a block; at its end the secondaries that reach the candidate threshold of the maximum so far
+            // become a bit mask (a compare and an add-with-carry each) and go into the list of the re-score below.  A
+            // threshold that has moved above the maximum before the block leaves everything listed before below the
+            // final threshold: the list starts over.
             const int iters = (S + slots - 1) / slots;          // of the slot with the most secondaries (wave-uniform)
             uint2 a_next = acol[4 * min(s_first, S - 1)];
+            float thr = -INFINITY;
             auto scan_block = [&](int i0, auto tail) -> uint32_t {
                 float b2v[32];
 #pragma unroll
@@ -278,7 +301,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                     // the running maximum takes two scores at a time (all ordinary numbers or -inf here)
                     if (i & 1) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(m2) : "v"(m2), "v"(b2v[i - 1]), "v"(b2));
                 }
-                const float thr = m2 - margin2;
+                thr = candidate_threshold<D>(m2, table_err, filter_err, margin2);
                 uint32_t word = 0u;
 #pragma unroll
                 for (int i = 31; i >= 0; i--)       // word = 2 word + (score >= thr): iteration i ends up in bit i
@@ -294,7 +317,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 const float m_before = m2;
                 const bool whole = (slots - 1) + (i0 + 31) * slots < S;     // every slot has all 32 secondaries of this block
                 uint32_t bits = whole ? scan_block(i0, std::false_type{}) : scan_block(i0, std::true_type{});
-                if (m_before < m2 - margin2) cnt = 0;
+                if (m_before < thr) cnt = 0;
                 while (bits) {
                     const int i = __builtin_ctz(bits);
                     bits &= bits - 1u;
@@ -327,7 +350,7 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
         int bk = 0x7fffffff;
         if (search) {
             if (cnt > kSCap) brute = true;
-            const float thr2 = m2 - margin2;
+            const float thr2 = candidate_threshold<D>(m2, table_err, filter_err, margin2);
             int kcnt = 0;
             if (!brute) {
                 for (int i = 0; i < cnt; i++) {

@@ -185,6 +185,39 @@ def test_full_size_filter_equals_bruteforce():
     assert torch.equal(a["idx"][:, :, 1000:1256].cpu(), want["idx"]) and torch.equal(a["rq"][:, :, 1000:1256].cpu(), want["rq"])
 
 
+@pytest.mark.parametrize("S", [24, 96, 192])
+@pytest.mark.parametrize("dn", ["fp16", "bf16"])
+def test_filter_equals_bruteforce_where_scores_tie(S, dn):
+    """The candidate threshold follows the rounding of the scores to the cache dtype; inputs whose best scores share
+    one rounded value are where a threshold set too high would drop the winner.  Chunks next to codewords, halfway
+    between two codewords, sparse and widely scaled rows: the filtered search must pick what the exhaustive scan
+    picks (2 M chunks per case)."""
+    ops, dt = _ops(), DT[dn]
+    H, T, d_h = 8, 8192, 128
+    g = torch.Generator(device=DEV).manual_seed(1000 + S)
+    raw = torch.randn(H, S, 4, generator=g, device=DEV)
+    J, slack = ops.build_joint(raw, dt)
+    K = J.shape[1]
+
+    def rows_of(pick):
+        return torch.gather(J.float(), 1, pick[..., None].expand(-1, -1, 4)).reshape(H, T, d_h)
+
+    r1 = rows_of(torch.randint(0, K, (H, T * d_h // 4), generator=g, device=DEV))
+    r2 = rows_of(torch.randint(0, K, (H, T * d_h // 4), generator=g, device=DEV))
+    scale = torch.exp(torch.randn(1, H, T, 1, generator=g, device=DEV))
+    cases = {
+        "near_codeword": (r1 * (1 + 1e-3 * torch.randn(H, T, d_h, generator=g, device=DEV)))[None] * scale,
+        "between_two": ((r1 + r2) * 0.5)[None],
+        "sparse": torch.randn(1, H, T, d_h, generator=g, device=DEV) * (torch.rand(1, H, T, d_h, generator=g, device=DEV) < 0.3),
+        "scaled": torch.randn(1, H, T, d_h, generator=g, device=DEV) * scale ** 3,
+    }
+    for name, x in cases.items():
+        x = x.to(dt)
+        a = ops.quantize(x, J, slack, 4, algo=0)
+        b = ops.quantize(x, J, slack, 4, algo=1)
+        assert torch.equal(a["idx"], b["idx"]) and torch.equal(a["rq"], b["rq"]), name
+
+
 # ---------------------------------------------------------------- dense decode
 @pytest.mark.parametrize("S,b_r", CODEBOOKS)
 @pytest.mark.parametrize("dn", ["fp32", "fp16", "bf16"])
