@@ -124,7 +124,7 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
     of the same arithmetic, used by the tests).  use_fp8_codebook decodes with the joint tables rounded to
     float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache);
     with fp8_table_storage=True the kernel also keeps them as float8 in LDS (half the table footprint, two
-    conversions per gathered codeword; same results, 5-15 % slower on MI355X, where the decode is bound by
+    conversions per gathered codeword; same results, 6-12 % slower on MI355X, where the decode is bound by
     vector-ALU issue and not by LDS space).
     """
     if fp8_table_storage and not use_fp8_codebook:
