@@ -524,6 +524,7 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     p.xcd_remap = (!a->kv_len && !a->batch_order && ((a->B * a->H_kv) % 8) == 0) ? 1 : 0;
     p.tab_fp8 = a->fp8_table_storage ? 1 : 0;
     p.wide_range = a->wide_range ? 1 : 0;
+    p.no_lds_landing = a->force_generic == 2 ? 1 : 0;
     // 4 consecutive scales with one vector load: unit stride, aligned rows, and capacity rows readable
     const int salign = a->dtype == HQMQ_F32 ? 16 : 8;
     p.scale_vec = 1;
@@ -547,7 +548,7 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
     tm.stop = (hipEvent_t)a->stop_event;
     int rc = HQMQ_OK;
     bool handled = false;
-    if (p.scale_vec && !a->force_generic && a->softmax_scale > 0.f) {
+    if (p.scale_vec && a->force_generic != 1 && a->softmax_scale > 0.f) {
         rc = launch_attn_fast(p, a->main_bits, flags, grid, ((size_t)a->K.K + a->V.K) * 8, st, tm, &handled);
         if (rc) return rc;
     }

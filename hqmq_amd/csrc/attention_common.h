@@ -52,6 +52,7 @@ struct AttnParams {
     unsigned m_hkv, m_G, m_gz, m_gx, m_splits;
     int tab_fp8;    // both tables hold e4m3 numbers and the caller asks for float8 storage in LDS
     int wide_range; // scales or verbatim values of the cache may leave the fp16 range: layout-generic kernel only
+    int no_lds_landing; // keep the specialised kernels that hold their tiles in registers (testing, measurements)
 };
 
 __device__ __forceinline__ float load_any(const void *p, int dtype, int64_t i) {

@@ -14,6 +14,7 @@
 // carry radius code 0 in the planes, so they decode to zero; their verbatim values enter through extra MFMAs
 // that walk the sideband entry list (values + coordinates), never the flag plane.
 #include "attention_common.h"
+#include <cstdlib>
 
 namespace hqmq {
 
@@ -968,6 +969,376 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Plain 16+0 caches at d_h 128 with tables of at most 2304 codewords (s96_r4 and smaller): the variant whose loads
+// all land in LDS (global_load_lds: the data goes from memory to LDS without passing through registers).  Tables,
+// the query rows and the first half-step of every wavefront are requested in the prologue; from then on a wavefront
+// asks for its next half-step when the current one has arrived and its words have been read out of the slot, so one
+// half-step per wavefront is in flight while one is being worked on.  Measured on config 2 at 32k, planes read cold
+// from HBM: asking for more ahead (two or three half-steps, before or behind the barrier) floods the memory system,
+// and the half-steps that are needed first then arrive behind later ones (first half-step in at 4.4 us median and
+// 8.2 us at worst with three ahead, 3.2 / 4.4 us with one); kernel 15.0 - 15.9 us with two or three ahead, 13.2 us
+// with one (the register-tile kernel, which keeps two ahead in 40 registers: 15.0 us).
+// No tile lives in registers while in flight (111 registers against 145 - 256).  The compiler neither sees these
+// loads nor counts them: every wait is written by hand (s_waitcnt vmcnt(n) lets the n youngest requests stay
+// outstanding; requests complete in order), and the kernel has no other vector loads before its epilogue.
+// LDS: K table at 0, V table at 18432, 4 KB of query rows, then per wavefront two slots of
+// [256 B scales: K tokens 0..31, V tokens 0..31, the same again][K rows of 32 tokens, 2 KB][V rows, 2 KB].
+constexpr int kLdVTab = 2304 * 8;
+constexpr int kLdQ = 2 * kLdVTab;
+constexpr int kLdSlot0 = kLdQ + 4096;
+constexpr int kLdSlotBytes = 256 + 4096;
+
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// wait until at most `groups` (0..3) groups of five requests are outstanding
+__device__ __forceinline__ void wait_groups(int groups) {
+    if (groups >= 3) wait_vm<15>();
+    else if (groups == 2) wait_vm<10>();
+    else if (groups == 1) wait_vm<5>();
+    else wait_vm<0>();
+}
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+}
+// 64 lanes x 16 bytes from base + voff (+ the instruction's offset, which counts for both sides) to LDS at m0 + 16 * lane
+__device__ __forceinline__ void lds_load16(uint32_t lds_base, const uint8_t *base, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_load16_addr(uint32_t lds_base, const uint8_t *addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(addr) : "memory");
+}
+__device__ __forceinline__ uint4v lds_read16(uint32_t a) { return *(lds_u4_ptr)(uintptr_t)a; }
+__device__ __forceinline__ uint2 lds_read8(uint32_t a) { return __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)a); }
+
+#ifdef HQMQ_STAMPS
+__device__ unsigned long long *g_stamps;
+#define STAMP(i) do { st_[i] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define STAMP(i) do { } while (0)
+#endif
+
+constexpr int kLdDepth = 2;
+
+template <int DT, int IB, int WV>
+__global__ __launch_bounds__(WV * 64) void attn_lds_kernel(AttnParams p) {
+    constexpr int CPL = 8, NW = 4, d_h = 128, mrb = 64;
+    extern __shared__ uint2 lds_tab[];
+#ifdef HQMQ_STAMPS
+    unsigned long long st_[16] = {};
+#endif
+    STAMP(0);
+    touch_kernargs();
+    // Everything the first requests need is read from the argument block in one go (the empty asm below is where
+    // all of it has to be there): read where it is used, every group of arguments costs its own round trip.
+    // The grid is (n_splits, column groups, B * Hkv): taken from the arguments, which spares the dispatch packet.
+    const unsigned gx = (unsigned)p.n_splits, gy = (unsigned)p.n_cg, gz = (unsigned)(p.B * p.Hkv);
+    const int Hkv = p.Hkv, remap = p.xcd_remap;
+    const unsigned m_gz = p.m_gz, m_gx = p.m_gx, m_hkv = p.m_hkv;
+    const int32_t *order_p = p.batch_order, *len_p = p.kv_len, *start_p = p.kv_start;
+    const uint8_t *kj = (const uint8_t *)p.Kc.joint, *vj = (const uint8_t *)p.Vc.joint;
+    const int64_t kjsh = p.Kc.jsh, vjsh = p.Vc.jsh;
+    const int KK = p.Kc.K, KV = p.Vc.K, Tkv = p.Tkv, Bn = p.B;
+    asm volatile("" ::"s"(gx), "s"(gy), "s"(gz), "s"(Hkv), "s"(remap), "s"(m_gz), "s"(m_gx), "s"(m_hkv), "s"(order_p), "s"(len_p), "s"(start_p),
+                 "s"(kj), "s"(vj), "s"(kjsh), "s"(vjsh), "s"(KK), "s"(KV), "s"(Tkv), "s"(Bn));
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    if (remap) {
+        const unsigned lin = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+        const unsigned r = fast_div(lin, gz, m_gz);
+        bz = (int)(lin - r * gz);
+        by = (int)fast_div(r, gx, m_gx);
+        bx = (int)(r - (unsigned)by * gx);
+    }
+    const int slot = (int)fast_div((unsigned)bz, (unsigned)Hkv, m_hkv), hkv = bz - slot * Hkv;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#ifdef HQMQ_STAMPS
+    asm volatile("" ::"s"(hkv));
+    STAMP(15);
+#endif
+    // the per-sequence words of ragged batches are read before the first request goes out: behind one, the wait for
+    // such a word would also wait for every request in flight
+    const int b = order_p ? min(max(order_p[slot], 0), Bn - 1) : slot;
+    int kv_end = len_p ? len_p[b] : Tkv;
+    kv_end = min(max(kv_end, 0), Tkv);
+    const int kv_first = start_p ? max(start_p[b], 0) : 0;
+    // ---- tables: 1 KB units dealt to the wavefronts round-robin, straight to their place in LDS ----
+    {
+        const uint32_t kbytes = (uint32_t)KK * 8u, vbytes = (uint32_t)KV * 8u;
+        const uint8_t *ksrc = uniform_ptr(kj + (size_t)hkv * kjsh * 2);
+        const uint8_t *vsrc = uniform_ptr(vj + (size_t)hkv * vjsh * 2);
+        const int ku = (int)((kbytes + 1023u) >> 10), nu = ku + (int)((vbytes + 1023u) >> 10);
+        for (int u = wave; u < nu; u += WV) {
+            const bool isv = u >= ku;
+            const uint32_t uu = (uint32_t)(isv ? u - ku : u);
+            const uint32_t off = min(uu * 1024u + (uint32_t)lane * 16u, (isv ? vbytes : kbytes) - 16u);      // past the end: the last pair again
+            lds_load16((isv ? (uint32_t)kLdVTab : 0u) + uu * 1024u, isv ? vsrc : ksrc, off);
+        }
+    }
+    STAMP(1);
+    const int bh = b * p.Hkv + hkv;
+    const int cg = by, sp = bx;
+    const int G = p.G;
+    const int col = lane & 15, grp = lane >> 4;
+    const int ncols = min(16, p.Tq * G - cg * 16);
+    const int cidx = cg * 16 + col;
+    const bool col_ok = col < ncols;
+    const int tq = col_ok ? (int)fast_div((unsigned)cidx, (unsigned)G, p.m_G) : 0;
+    int col_lim, blk_lim, lim_min;
+    {
+        int64_t lim64 = kv_end;
+        if (p.causal) lim64 = min(lim64, (int64_t)tq + p.causal_offset + 1);
+        if (!col_ok || lim64 < 0) lim64 = 0;
+        col_lim = (int)lim64;
+        blk_lim = col_lim;
+        lim_min = col_ok ? col_lim : 0x7fffffff;
+    }
+    if (p.causal) {
+        for (int o = 1; o < 16; o <<= 1) {
+            blk_lim = max(blk_lim, __shfl_xor(blk_lim, o));
+            lim_min = min(lim_min, __shfl_xor(lim_min, o));
+        }
+        blk_lim = __builtin_amdgcn_readfirstlane(blk_lim);
+        lim_min = __builtin_amdgcn_readfirstlane(lim_min);
+    } else {
+        blk_lim = lim_min = kv_end;
+    }
+    const int col_start = min(kv_first, blk_lim);
+    const int blk_lo = col_start / kSuper * kSuper;
+    int per_split = (int)fast_div((unsigned)(blk_lim - blk_lo + p.n_splits - 1), (unsigned)p.n_splits, p.m_splits);
+    per_split = (per_split + kSuper - 1) / kSuper * kSuper;
+    const int b_begin = min(blk_lo + sp * per_split, blk_lim), b_end = min(blk_lim, b_begin + per_split);
+    constexpr int TS = 32 * WV;
+    const int t_begin = min(b_begin + wave * 32, b_end), t_end = b_end;
+    const int n_hs = __builtin_amdgcn_readfirstlane(t_begin < t_end ? (t_end - t_begin + TS - 1) / TS : 0);
+    const size_t plane_row0 = (size_t)bh * p.t_cap;
+    const int idx_bits = p.idx_bits;
+    // instruction offsets count for the memory and the LDS side alike: the bases are moved back by the slot offsets
+    const uint8_t *k_rows = p.Kc.main_plane + plane_row0 * mrb - 256;
+    const uint8_t *v_rows = p.Vc.main_plane + plane_row0 * mrb - 2304;
+    const uint32_t main_off = (uint32_t)(col * mrb + grp * 16);
+    // scales: lanes 0..15 fetch the K scales of tokens 2 lane, 2 lane + 1, lanes 16..31 the V scales; the upper half repeats
+    const uint8_t *sc_lane = (lane & 16) ? (const uint8_t *)((const uint16_t *)p.Vc.scale_plane + b * p.Vc.ssb + hkv * p.Vc.ssh)
+                                         : (const uint8_t *)((const uint16_t *)p.Kc.scale_plane + b * p.Kc.ssb + hkv * p.Kc.ssh);
+    sc_lane += 4 * (lane & 15);
+    const uint32_t slot_base = (uint32_t)(kLdSlot0 + wave * kLdDepth * kLdSlotBytes);
+    auto request = [&](int th, uint32_t slot_lds) {
+        const uint8_t *kb = uniform_ptr(k_rows + (size_t)th * mrb), *vb = uniform_ptr(v_rows + (size_t)th * mrb);
+        const uint8_t *sa = sc_lane + 2 * (size_t)th;
+        asm volatile("s_mov_b32 m0, %0\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:256\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:1280\n\t"
+                     "global_load_lds_dword %1, off\n\t"
+                     "global_load_lds_dwordx4 %2, %4 offset:2304\n\t"
+                     "global_load_lds_dwordx4 %2, %4 offset:3328"
+                     ::"s"(slot_lds), "v"(sa), "v"(main_off), "s"(kb), "s"(vb) : "memory");
+    };
+    // ---- query rows (first wavefront): column c of the block at kLdQ + 256 c, raw 16-bit values ----
+    if (wave == 0) {
+        for (int i = 0; 4 * i < ncols; i++) {       // four columns per request; a decode step of G <= 4 heads takes one
+            const int c = min(4 * i + (lane >> 4), ncols - 1);              // lanes past the last real column repeat it (never read)
+            const int ci = cg * 16 + c;
+            const int tqc = (int)fast_div((unsigned)ci, (unsigned)G, p.m_G), hqc = hkv * G + (ci - tqc * G);
+            const uint8_t *qa = (const uint8_t *)((const uint16_t *)p.Q + b * p.qsb + hqc * p.qsh + (int64_t)tqc * p.qst) + 16 * (lane & 15);
+            lds_load16_addr((uint32_t)(kLdQ + 1024 * i), qa);
+        }
+    }
+    // the first half-step; the later ones are requested from inside the loop, one ahead
+    if (n_hs > 0) request(t_begin, slot_base);
+    STAMP(2);
+    half4 ident;
+#pragma unroll
+    for (int e = 0; e < 4; e++) ident[e] = (_Float16)((4 * grp + e) == col ? 1.f : 0.f);
+    wait_groups(n_hs > 0 ? 1 : 0);            // tables (and query rows) in: only the tile request may still be outstanding
+    STAMP(3);
+    asm volatile("s_barrier" ::: "memory");
+    if constexpr (DT != HQMQ_F16) {
+        // the tables landed in the cache dtype: converted to fp16 in place, two codewords per thread and round
+        for (int k = threadIdx.x; k < (2 * kLdVTab) / 16; k += WV * 64) {
+            const uint4v w = pair_to_half<DT>(lds_read16((uint32_t)k * 16u));
+            *(uint4v __attribute__((address_space(3))) *)(uintptr_t)((uint32_t)k * 16u) = w;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);         // lgkmcnt(0): the stores are in LDS
+        asm volatile("s_barrier" ::: "memory");
+    }
+    STAMP(4);
+    half8 qf[CPL / 2];
+#pragma unroll
+    for (int j = 0; j < CPL / 2; j++) {
+        const uint4v w = lds_read16((uint32_t)(kLdQ + col * 256 + grp * 64 + 16 * j));
+        const half4 lo = chunk_to_half<DT>(uint2{w[0], w[1]}), hi = chunk_to_half<DT>(uint2{w[2], w[3]});
+        const half4 z = half4{0, 0, 0, 0};
+        qf[j] = cat8(col_ok ? lo : z, col_ok ? hi : z);
+    }
+
+    const float c = p.c_log2;
+    float m_run = -INFINITY, l_run = 0.f;
+    float4v acc[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; j++) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
+    int ring = 0;
+    for (int i = 0, th = t_begin; i < n_hs; i++, th += TS) {
+        const uint32_t sl = slot_base + (uint32_t)ring * kLdSlotBytes, sl_next = slot_base + (uint32_t)(ring ^ 1) * kLdSlotBytes;
+        ring ^= 1;
+        wait_groups(0);
+#ifdef HQMQ_STAMPS
+        { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime();
+          if (i == 0) st_[5] = t_; else if (i == 1) st_[7] = t_; else if (i == 2) st_[9] = t_; else if (i == 3) st_[11] = t_; }
+#endif
+        uint4v kw[2], vw[2];
+        uint2 ks[2], vs[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            kw[u] = lds_read16(sl + 256u + 1024u * u + 16u * (uint32_t)lane);
+            ks[u] = lds_read8(sl + 32u * u + 8u * (uint32_t)grp);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            vw[u] = lds_read16(sl + 2304u + 1024u * u + 16u * (uint32_t)lane);
+            vs[u] = lds_read8(sl + 64u + 32u * u + 8u * (uint32_t)grp);
+        }
+        // the words of this half-step are in registers: ask for the next one (into the other slot)
+        asm volatile("" : "+v"(kw[0]), "+v"(kw[1]), "+v"(vw[0]), "+v"(vw[1]), "+v"(ks[0]), "+v"(ks[1]), "+v"(vs[0]), "+v"(vs[1]));
+        if (i + 1 < n_hs) request(th + TS, sl_next);
+
+        float4v sT[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            half4 g[CPL], a[CPL];
+            half2v r[CPL / 2];
+            const uint32_t w[NW] = {kw[u][0], kw[u][1], kw[u][2], kw[u][3]};
+            gather_chunks<CPL, 16, 0, IB, NW, 0, false>(w, 0u, idx_bits, g, r);
+            scale_chunks<CPL, false>(g, r, a);
+            float4v s = zero4;
+#pragma unroll
+            for (int jj = 0; jj < CPL / 2; jj++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(a[2 * jj], a[2 * jj + 1]), qf[jj], s, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s[e] = scaled<DT>(s[e], e < 2 ? ks[u].x : ks[u].y, e & 1, 0.f);
+            sT[u] = s;
+        }
+        const bool edge = !(th + 32 <= lim_min && th + 32 <= t_end && th >= col_start);
+        if (edge) {
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int t = th + 16 * u + 4 * grp + e;
+                    if (!(t < col_lim && t < t_end && t >= col_start)) sT[u][e] = -INFINITY;
+                }
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(sT[0][0], sT[0][1]), fmaxf(sT[0][2], sT[0][3])), fmaxf(fmaxf(sT[1][0], sT[1][1]), fmaxf(sT[1][2], sT[1][3])));
+        tmax = row_max4(tmax);
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+            l_run *= alpha;
+#pragma unroll
+            for (int j = 0; j < CPL; j++) acc[j] = acc[j] * alpha;
+            m_run = m_new;
+        }
+        const float mc = -m_use * c;
+        half4 pT[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            float pe[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                pe[e] = __builtin_amdgcn_exp2f(fmaf(sT[u][e], c, mc));
+                l_run += pe[e];
+            }
+            const half2v p01 = half2v{(_Float16)pe[0], (_Float16)pe[1]} * scale_h2<DT>(vs[u].x);
+            const half2v p23 = half2v{(_Float16)pe[2], (_Float16)pe[3]} * scale_h2<DT>(vs[u].y);
+            pT[u] = half4{p01[0], p01[1], p23[0], p23[1]};
+        }
+        const half8 pp = cat8(pT[0], pT[1]);
+        half4 av[2][CPL];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            half4 g[CPL];
+            half2v r[CPL / 2];
+            const uint32_t w[NW] = {vw[u][0], vw[u][1], vw[u][2], vw[u][3]};
+            gather_chunks<CPL, 16, 0, IB, NW, kLdVTab, false>(w, 0u, idx_bits, g, r);
+            scale_chunks<CPL, false>(g, r, av[u]);
+        }
+#pragma unroll
+        for (int j = 0; j < CPL; j++) {
+            const float4v t0v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[0][j], ident, zero4, 0, 0, 0);
+            const float4v t1v = __builtin_amdgcn_mfma_f32_16x16x16f16(av[1][j], ident, zero4, 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cat8(pack4(t0v), pack4(t1v)), pp, acc[j], 0, 0, 0);
+        }
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(acc[0]), "v"(acc[7]));
+        { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime();
+          if (i == 0) st_[6] = t_; else if (i == 1) st_[8] = t_; else if (i == 2) st_[10] = t_; else if (i == 3) st_[12] = t_; }
+#endif
+    }
+
+    // ---- merge the block's wavefronts through LDS: rows of [d_h accumulators, m, l, pad] ----
+    constexpr int RS = d_h + 4, NT = WV * 64;
+    float *red = reinterpret_cast<float *>(lds_tab);
+    const float inv_qmax = p.inv_qmax;
+    const float l_tot = row_sum4(l_run);
+    __syncthreads();
+    if (col < ncols) {
+        float *wp = red + ((size_t)wave * 16 + col) * RS;
+        if (grp == 0) { wp[d_h] = m_run; wp[d_h + 1] = l_tot; }
+#pragma unroll
+        for (int j = 0; j < CPL; j++) *reinterpret_cast<float4v *>(wp + grp * CPL * 4 + 4 * j) = acc[j];
+    }
+    __syncthreads();
+    STAMP(13);
+    for (int o = threadIdx.x; o < ncols * d_h; o += NT) {
+        const int cc = o / d_h, e = o - cc * d_h;
+        const int ci = cg * 16 + cc;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WV; w++) m = fmaxf(m, red[((size_t)w * 16 + cc) * RS + d_h]);
+        float l = 0.f, a = 0.f;
+        if (m > -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < WV; w++) {
+                const float *q = red + ((size_t)w * 16 + cc) * RS;
+                const float f = __builtin_amdgcn_exp2f((q[d_h] - m) * c);
+                l = fmaf(q[d_h + 1], f, l);
+                a = fmaf(q[e], f, a);
+            }
+        }
+        const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
+        if (p.n_splits == 1) {
+            store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
+        } else {
+            float *wp = p.ws + ((((size_t)b * p.Hq + hq2) * p.Tq + tq2) * p.n_splits + sp) * (size_t)(d_h + kPartialHead);
+            if (e == 0) { wp[0] = m * c; wp[1] = l; }
+            wp[kPartialHead + e] = a * inv_qmax;
+        }
+    }
+#ifdef HQMQ_STAMPS
+    STAMP(14);
+    if (lane == 0 && g_stamps) {
+        unsigned long long *o = g_stamps + ((size_t)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * WV + wave) * 16;
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[i] = st_[i];
+    }
+#endif
+}
+
+template <int DT, int IB>
+static int launch_lds(const AttnParams &p, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
+    constexpr int WV = kFastWaves;
+    constexpr size_t kTiles = (size_t)kLdSlot0 + (size_t)WV * kLdDepth * kLdSlotBytes;
+    constexpr size_t kMerge = (size_t)WV * 16 * (128 + 4) * sizeof(float);
+    constexpr size_t shmem = kTiles > kMerge ? kTiles : kMerge;
+    static_assert(shmem <= 160 * 1024, "LDS of one CU");
+    auto kern = attn_lds_kernel<DT, IB, WV>;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (e != hipSuccess) return (int)e;
+    launch_timed(kern, grid, dim3(WV * 64), shmem, st, tm, p);
+    return hip_status(hipGetLastError());
+}
+
 template <int CPL, int MB, int AB, int IB, int DT, int WV = kFastWaves, int NCG = 1, bool F8 = false>
 static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm) {
     if (NCG > 1) grid.y = (grid.y + NCG - 1) / NCG;
@@ -1006,6 +1377,12 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
         if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) return launch_one<8, 16, 0, 12, DT, kFastWaves, 1, true>(p, flags, grid, st, tm);
         if (mb == 16 && p.aux_bits == 3 && p.idx_bits == 13 && p.Kc.K <= 4608) return launch_one<8, 16, 3, 13, DT, kFastWaves, 1, true>(p, flags, grid, st, tm);
     }
+    // plain 16+0 caches with small tables at d_h 128, one column group, eight wavefronts: every load lands in LDS
+    if constexpr (CPL == 8) {
+        if (mb == 16 && p.aux_bits == 0 && !flags && !two && !wide && !p.no_lds_landing && p.Kc.K <= 2304 && p.Vc.K <= 2304 && p.Kc.K >= 2 &&
+            p.Vc.K >= 2 && ((((uintptr_t)p.Q) | (uintptr_t)(p.qsb * 2) | (uintptr_t)(p.qsh * 2) | (uintptr_t)(p.qst * 2)) & 15) == 0)
+            return p.idx_bits == 12 ? launch_lds<DT, 12>(p, grid, st, tm) : launch_lds<DT, 0>(p, grid, st, tm);
+    }
     if (mb == 16 && p.aux_bits == 0 && p.idx_bits == 12) {
         if (two) return launch_one<CPL, 16, 0, 12, DT, kFastWaves, 2>(p, flags, grid, st, tm);
         return wide ? launch_one<CPL, 16, 0, 12, DT, 12>(p, flags, grid, st, tm) : launch_one<CPL, 16, 0, 12, DT>(p, flags, grid, st, tm);
@@ -1039,6 +1416,10 @@ static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hip
     *handled = false;
     return HQMQ_OK;
 }
+
+#ifdef HQMQ_STAMPS
+extern "C" int hqmq_debug_set_stamps(void *ptr) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_stamps), &ptr, sizeof(ptr)); }
+#endif
 
 int launch_attn_fast(const AttnParams &p, int main_bits, bool flags, dim3 grid, size_t table_bytes, hipStream_t st,
                      const LaunchTiming &tm, bool *handled) {
