@@ -396,6 +396,45 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const flo
     }
 }
 
+// The same merge for the common decode shape (d_h = 128, at most 32 splits, 16-bit output): one wavefront per row and
+// no LDS.  A lane owns two output elements and loads them from all 32 split records at once (8 bytes each, 512 bytes
+// per wavefront and record), together with the (m, l) pair of split (lane & 31): one round trip to memory.  The
+// maximum and the denominator are reduced across the lanes, the 32 weights are read back lane by lane into scalar
+// registers and multiply the records in place.
+__global__ __launch_bounds__(64) void attn_combine_wave_kernel(const float *__restrict__ ws, uint16_t *__restrict__ O, int dtype, int Hq, int Tq,
+                                                              int n_splits, int64_t osb, int64_t osh, int64_t ost) {
+    constexpr int d_h = 128, rec = d_h + kPartialHead, NS = 32;
+    const unsigned row = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float *base = ws + (size_t)row * (size_t)n_splits * rec;
+    const int sl = lane & 31;
+    float2 ml = *reinterpret_cast<const float2 *>(base + (size_t)min(sl, n_splits - 1) * rec);
+    float2 as[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) as[s] = *reinterpret_cast<const float2 *>(base + (size_t)min(s, n_splits - 1) * rec + kPartialHead + 2 * lane);
+    if (sl >= n_splits) ml = float2{-INFINITY, 0.f};
+    float M = ml.x;
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
+    const float w = M > -INFINITY ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;        // -inf - finite = -inf -> 0
+    float L = ml.y * w;
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) L += __shfl_xor(L, o);
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const float wsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s));
+        a0 = fmaf(as[s].x, wsc, a0);
+        a1 = fmaf(as[s].y, wsc, a1);
+    }
+    const float r0 = L > 0.f ? a0 / L : 0.f, r1 = L > 0.f ? a1 / L : 0.f;
+    const unsigned bh = row / (unsigned)Tq, tq = row - bh * (unsigned)Tq, b = bh / (unsigned)Hq, hq = bh - b * (unsigned)Hq;
+    const int64_t o = (int64_t)b * osb + (int64_t)hq * osh + (int64_t)tq * ost + 2 * lane;
+    const uint32_t h0 = dtype == HQMQ_F16 ? __half_as_ushort(__float2half_rn(r0)) : f32_to_bf16_bits(r0);
+    const uint32_t h1 = dtype == HQMQ_F16 ? __half_as_ushort(__float2half_rn(r1)) : f32_to_bf16_bits(r1);
+    *reinterpret_cast<uint32_t *>(O + o) = h0 | h1 << 16;
+}
+
 static PackedDev to_dev(const hqmq_packed &k) {
     return PackedDev{k.main_plane, k.aux_plane, k.flag_plane, k.scale_plane, k.scale_sb, k.scale_sh, k.scale_st,
                      k.sideband, k.sb_tile_off, k.sb_cap, k.sb_coord, k.sb_count, k.joint, k.joint_sh, k.K, k.scale_max_bits};
@@ -458,6 +497,11 @@ extern "C" int hqmq_attn_combine(const void *workspace, void *O, int dtype, int 
     const int64_t rows = (int64_t)B * H_q * T_q;
     if (rows > 0x7fffffff) return HQMQ_ERR_SHAPE;
     if ((uintptr_t)workspace & 15) return HQMQ_ERR_ALIGN;
+    if (d_h == 128 && n_splits <= 32 && dtype != HQMQ_F32 && ((((uintptr_t)O) | (uintptr_t)(o_sb * 2) | (uintptr_t)(o_sh * 2) | (uintptr_t)(o_st * 2)) & 3) == 0) {
+        hipLaunchKernelGGL(attn_combine_wave_kernel, dim3((unsigned)rows), dim3(64), 0, (hipStream_t)stream, (const float *)workspace,
+                           (uint16_t *)O, dtype, H_q, T_q, n_splits, o_sb, o_sh, o_st);
+        return hip_status(hipGetLastError());
+    }
     hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)rows), dim3(kCombineThreads), 0, (hipStream_t)stream,
                        (const float *)workspace, O, dtype, H_q, T_q, d_h, n_splits, o_sb, o_sh, o_st);
     return hip_status(hipGetLastError());
