@@ -110,7 +110,7 @@ LAST_KERNEL_STATS = {}
 
 
 def kernel_time_us(launch, iters):
-    """Average GPU duration of the attention kernel itself over `iters` launches launch(i, events): every launch
+    """Median GPU duration of the attention kernel itself over `iters` launches launch(i, events): every launch
     carries its own pair of HIP events, which the runtime stamps at the begin and at the end of that dispatch (the
     same interval a kernel trace reports; the gap between two dependent dispatches is not part of it)."""
     import ctypes as C
@@ -134,12 +134,14 @@ def kernel_time_us(launch, iters):
         durs.append(ms.value * 1e3)
         hip.hipEventDestroy(a)
         hip.hipEventDestroy(b)
-    # eager launches are paced by the host: now and then one is stretched by whatever else the device was doing between
-    # them.  Launches beyond 1.5 x the median are left out of the average; LAST_KERNEL_STATS keeps the full picture.
+    # The median of all launches is what is reported (eager launches are paced by the host, and now and then one is
+    # stretched by whatever else the device did between them); the plain mean, the maximum and the mean without the
+    # launches beyond 1.5 x the median go into LAST_KERNEL_STATS, nothing is left out of the figure itself.
     med = sorted(durs)[len(durs) // 2]
     kept = [d for d in durs if d <= 1.5 * med]
-    LAST_KERNEL_STATS.update(mean_all=sum(durs) / len(durs), median=med, max=max(durs), dropped=len(durs) - len(kept))
-    return sum(kept) / len(kept)
+    LAST_KERNEL_STATS.update(mean_all=sum(durs) / len(durs), median=med, max=max(durs), min=min(durs),
+                             mean_without_stretched=sum(kept) / len(kept), stretched=len(durs) - len(kept), launches=len(durs))
+    return med
 
 
 def cpu_attention_baseline(slice_tokens, repeats=5):
@@ -166,27 +168,70 @@ def cpu_attention_baseline(slice_tokens, repeats=5):
     return times[len(times) // 2]
 
 
+def config1_inputs():
+    """Benchmark config 1: K and V of one layer, Mistral-7B shape (8 KV heads, d_h 128, batch 1, 2048 tokens), fp16
+    ~N(0,1) with lognormal(0, 0.5) channel scales; CPU-seeded, the same tensors for the GPU and the CPU leg."""
+    import torch
+    from tests.helpers import kv_input
+    return kv_input((1, 8, 2048, 128), torch.float16, 1), kv_input((1, 8, 2048, 128), torch.float16, 2)
+
+
 def cpu_quantize_baseline_config1(repeats=3):
-    """Benchmark config 1 in full on the host: K and V of one layer (8 heads, 2048 tokens, d_h 128, fp16 with
-    lognormal channel scales), s24_r3 with Med3x (C = 3): the restated reference quantizer, median of `repeats`
-    after one warm-up.  Returns (seconds for K and V, tokens)."""
+    """Benchmark config 1 in full on the host: s24_r3 with Med3x (C = 3), the restated reference quantizer
+    (reference: src/quantizers/hqmq.py:145-216, outlier_aware.py:56-87), median of `repeats` after one warm-up.
+    Returns (seconds for K and V, tokens, MSE of the dequantized K and V against the input)."""
     import torch
     from oracle import torch_oracle as TO
-    from tests.helpers import kv_input
-    dt, T = torch.float16, 2048
-    k, v = kv_input((1, 8, T, 128), dt, 1), kv_input((1, 8, T, 128), dt, 2)
+    k, v = config1_inputs()
+    T = k.shape[2]
     raw = TO.secondary_raw(1, 8, 24, 42)
-    Jk, Jv = TO.joint_table(raw[0, :, 0], dt), TO.joint_table(raw[0, :, 1], dt)
-    times = []
+    Jk, Jv = TO.joint_table(raw[0, :, 0], k.dtype), TO.joint_table(raw[0, :, 1], k.dtype)
+    times, mse = [], None
     for i in range(1 + repeats):
         t0 = time.perf_counter()
-        TO.outlier_quantize(k, Jk, 3, 3.0)
-        TO.outlier_quantize(v, Jv, 3, 3.0)
+        rk = TO.outlier_quantize(k, Jk, 3, 3.0)
+        rv = TO.outlier_quantize(v, Jv, 3, 3.0)
         dtm = time.perf_counter() - t0
         if i >= 1:
             times.append(dtm)
+        mse = (float(((rk["out"].float() - k.float()) ** 2).mean()), float(((rv["out"].float() - v.float()) ** 2).mean()))
     times.sort()
-    return times[len(times) // 2], T
+    return times[len(times) // 2], T, mse
+
+
+def gpu_config1(dev, calls=10):
+    """Benchmark config 1 on the GPU: quantize + Med3x (C = 3) + pack of K and V of one layer into a packed cache
+    (one bulk append), then the dequantized KV and its MSE against the input, outlier rate and bits per value."""
+    import torch
+    import hqmq
+    from hqmq_amd import ops
+    k, v = config1_inputs()
+    k, v = k.to(dev), v.to(dev)
+    T, d = k.shape[2], k.shape[3]
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=8, secondary_size=24, radius_bits=3, device=dev), C=3.0)
+    fresh = [w.new_cache(1, T, d, k.dtype, 0) for _ in range(calls + 3)]
+    for c in fresh[:3]:
+        w.append(c, k, v, 0)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for c in fresh[3:]:
+        w.append(c, k, v, 0)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / calls
+    cache = fresh[-1]
+    cache.K.check_overflow()
+    cache.V.check_overflow()
+    Kd, Vd = ops.dequant_packed(cache.K, T, 0), ops.dequant_packed(cache.V, T, 0)
+    chunks = 8 * T * d // 4
+    return {"what": "BASELINE config 1 on the GPU: one bulk append = quantize (s24_r3) + Med3x (C = 3) + bit-packing + sideband of K and V, "
+                    "8 heads x 2048 tokens x d_h 128 fp16; MSE of the cache dequantized again (packed codes + verbatim outlier chunks) "
+                    "against the input",
+            "us_per_call_K_and_V": round(us, 1), "GTok_per_s": round(T / us / 1e3, 6),
+            "mse_K": float(((Kd.float() - k.float()) ** 2).mean()), "mse_V": float(((Vd.float() - v.float()) ** 2).mean()),
+            "outlier_rate_K": round(float(cache.K.sb_count.sum()) / chunks, 5), "outlier_rate_V": round(float(cache.V.sb_count.sum()) / chunks, 5),
+            "bits_per_value": round(w.bits_per_value(), 4), "packed_bytes_K_and_V": cache.nbytes(T)}
 
 
 def main():
@@ -284,11 +329,11 @@ def main():
     us_step_same, _ = graph_us(step_same, args.steps, stream)
     achieved = cache_bytes / (us_main * 1e-6) / 1e9
     # what the memory system allows a launch of this shape: the kernel that only reads the same planes with the same
-    # grid, per-wavefront ranges and loads (hqmq_attn_read_ceiling), caches rotating / one cache
-    us_read = kernel_time_us(lambda i, ev: ops.read_ceiling(caches[i % NL].K, caches[i % NL].V, T, H_q=Hq, n_splits=n_splits,
-                                                             depth=3, waves=8, kernel_events=ev), 192)
-    us_read_same = kernel_time_us(lambda i, ev: ops.read_ceiling(caches[0].K, caches[0].V, T, H_q=Hq, n_splits=n_splits,
-                                                                  depth=3, waves=8, kernel_events=ev), 192)
+    # grid, per-wavefront ranges and loads (libhqmq_bench.so: hqmq_bench_read_planes), caches rotating / one cache
+    from hqmq_amd import bench_ceiling
+    sink = torch.empty(1 << 22, dtype=torch.uint8, device=dev)
+    us_read = kernel_time_us(lambda i, ev: bench_ceiling.read_planes(caches[i % NL], n_splits, 3, 8, ev, sink), 192)
+    us_read_same = kernel_time_us(lambda i, ev: bench_ceiling.read_planes(caches[0], n_splits, 3, 8, ev, sink), 192)
 
     result = {
         "metric": "decode-attn HBM GB/s on compressed bytes (us/step and % of 8 TB/s alongside); quantize GTok/s",
@@ -316,7 +361,7 @@ def main():
                      "traffic": RECORDED_TRAFFIC_BYTES.get(T),
                      "traffic_source": f"{TRAFFIC_FILE} (FETCH_SIZE + WRITE_SIZE of an earlier rocprofv3 --pmc run; not "
                                        f"measured by this run)" if T in RECORDED_TRAFFIC_BYTES else None,
-                     "kernel": "hqmq::attn_fast_kernel<8, 16, 0, 12, 1, false, 8, 1, false>", "kernel_us": round(us_main, 2), "kernel_us_stats": main_stats,
+                     "kernel": "hqmq::attn_lds_kernel<1, 12, 8>", "kernel_us": round(us_main, 2), "kernel_us_is": "median of 192 launches, each with its own pair of HIP events", "kernel_us_stats": main_stats,
                      "kernel_launch_interval_us": round(us_launch_interval, 2),
                      "algorithmic_bytes_per_launch": cache_bytes,
                      "read_only_kernel_same_grid_us": round(us_read, 2),
@@ -338,8 +383,18 @@ def main():
             c2.K.length = c2.V.length = 0
             q.append(c2, k, v, 0)
         us_quant = event_time_us(quant_only, 10, stream)
+        # algorithmic bytes of the call: K and V, 8 heads: the input row (d_h x 2 B) read, the packed row (66 B) written
+        q_bytes = 2 * Hkv * T * (D_H * 2 + cache_bytes // (2 * Hkv * T))
+        valu_per_wave, waves = 1885, 2 * Hkv * T * (D_H // 4) // 64       # instructions per wavefront of 64 chunks: recorded by rocprofv3
         result["quantize"] = {"GTok_per_s": round(T / (us_quant * 1e-6) / 1e9, 5), "us_per_call": round(us_quant, 1), "tokens": T,
-                              "what": "K and V of one layer, 8 kv heads x d_h 128, s96_r4 fp16, quantize + pack"}
+                              "what": "K and V of one layer, 8 kv heads x d_h 128, s96_r4 fp16, quantize + pack (no Med3x); "
+                                      "the config-1 workload (s24_r3 + Med3x) is in the config1 block, GPU and CPU on the same input",
+                              "algorithmic_bytes_per_call": q_bytes, "GBps": round(q_bytes / us_quant / 1e3, 1),
+                              "bytes_roofline_frac": round(q_bytes / us_quant / 1e3 / HBM_PEAK_GBPS, 4),
+                              "valu_issue_frac": round(valu_per_wave * 4 * waves / (1024 * 2.4e3 * us_quant), 3),
+                              "valu_issue_frac_is": "1,885 vector-ALU instructions per wavefront (profiles/quantize_kernel_s96r4_fp16_32k.txt, "
+                                                    "recorded offline) x 4 cycles x wavefronts / (1024 SIMDs x 2.4 GHz x the measured time): "
+                                                    "the kernel is bound by vector-ALU issue, not by bytes"}
         k1, v1 = k[:, :, :1].contiguous(), v[:, :, :1].contiguous()
 
         def append_one(i):
@@ -391,12 +446,18 @@ def main():
             r = bench_configs.run(cfg, 30, emit=False)
             result["configs_3_4_5"][str(cfg)] = r
             torch.cuda.empty_cache()
+    if not args.quick:
+        result["config1"] = gpu_config1(dev)
     if not args.no_cpu_baseline:
         threads = torch.get_num_threads()
         slice_tokens = 4096
         sec = cpu_attention_baseline(slice_tokens)
         slice_bytes = cache_bytes * slice_tokens / T
-        qsec, qtok = cpu_quantize_baseline_config1()
+        qsec, qtok, qmse = cpu_quantize_baseline_config1()
+        if "config1" in result:
+            result["config1"].update(cpu_us_per_call_K_and_V=round(qsec * 1e6, 1), cpu_GTok_per_s=round(qtok / qsec / 1e9, 8),
+                                     cpu_mse_K=qmse[0], cpu_mse_V=qmse[1], cpu_cores=threads,
+                                     cpu_what="the restated reference quantizer (oracle, torch on the host) on the same tensors")
         result["cpu_baseline"] = {
             "value": round(slice_bytes / sec / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"torch restatement of the reference path (dense decode + SDPA), fp16, {slice_tokens} of {T} tokens, "

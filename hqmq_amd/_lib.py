@@ -76,8 +76,9 @@ EXPORTS = [
     "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",
     "hqmq_pack_codes", "hqmq_dequant_packed", "hqmq_attn_workspace_bytes", "hqmq_attn_pick_splits",
     "hqmq_attn_fwd", "hqmq_attn_combine", "hqmq_append_kv", "hqmq_attn_static_scratch_bytes", "hqmq_attn_fwd_static",
-    "hqmq_attn_read_ceiling_sink_bytes", "hqmq_attn_read_ceiling",
 ]
+BENCH_EXPORTS = ["hqmq_bench_read_planes_sink_bytes", "hqmq_bench_read_planes", "hqmq_bench_read_plain", "hqmq_bench_read_lds",
+                 "hqmq_bench_empty"]
 
 
 def library_path() -> Path:
@@ -93,11 +94,26 @@ def lib():
         L = C.CDLL(str(_SO))
         L.hqmq_status_string.restype = C.c_char_p
         L.hqmq_status_string.argtypes = [C.c_int]
-        for name in ("hqmq_med3x_workspace_bytes", "hqmq_attn_workspace_bytes", "hqmq_attn_static_scratch_bytes",
-                     "hqmq_attn_read_ceiling_sink_bytes"):
+        for name in ("hqmq_med3x_workspace_bytes", "hqmq_attn_workspace_bytes", "hqmq_attn_static_scratch_bytes"):
             getattr(L, name).restype = i64
         _lib = L
     return _lib
+
+
+_bench_lib = None
+
+
+def bench_lib():
+    """The measurement library (read-only probe kernels); loaded by bench.py and hqmq_amd/bench_ceiling.py only."""
+    global _bench_lib
+    if _bench_lib is None:
+        so = _SO.with_name("libhqmq_bench.so")
+        if not so.exists():
+            raise HqmqError(f"{so} is missing: build it with `python -m hqmq_amd.build` (needs hipcc)")
+        L = C.CDLL(str(so))
+        L.hqmq_bench_read_planes_sink_bytes.restype = i64
+        _bench_lib = L
+    return _bench_lib
 
 
 def check(status: int, what: str) -> None:

@@ -120,8 +120,9 @@ def fused_attention_packed(Q: torch.Tensor, cache: PackedKV, *, causal: bool = F
     cached tokens before the chunk (bottom-right alignment).  Ragged batches pass kv_lens (int32 [B]);
     left-padded batches pass kv_starts (int32 [B], the first real token of every sequence).  batch_order (int32 [B],
     e.g. ops.longest_first(kv_lens)) starts the sequences' blocks in that order: scheduling only, same result.
-    force_generic runs the layout-generic kernel where a specialised one exists (a second implementation
-    of the same arithmetic, used by the tests).  use_fp8_codebook decodes with the joint tables rounded to
+    force_generic (True or 1) runs the layout-generic kernel where a specialised one exists (a second implementation
+    of the same arithmetic, used by the tests); 2 keeps the specialised kernels that hold their tiles in registers
+    where the one that lands its loads in LDS would run (plain 16+0 caches at d_h 128; same results bit for bit).  use_fp8_codebook decodes with the joint tables rounded to
     float8_e4m3fn (an accuracy/footprint experiment of the reference; the rounded tables are kept per cache);
     with fp8_table_storage=True the kernel also keeps them as float8 in LDS (half the table footprint, two
     conversions per gathered codeword; same results, 6-12 % slower on MI355X, where the decode is bound by

@@ -1,4 +1,6 @@
-"""Builds hqmq_amd/libhqmq_amd.so from hqmq_amd/csrc/*.hip with hipcc for gfx950.
+"""Builds hqmq_amd/libhqmq_amd.so from hqmq_amd/csrc/*.hip with hipcc for gfx950, and beside it
+hqmq_amd/libhqmq_bench.so from hqmq_amd/csrc_bench/*.hip: the read-only measurement kernels that bench.py and
+hqmq_amd/bench_ceiling.py time (nothing in the product path loads that one).
 
     python -m hqmq_amd.build            # compile (always) and link
 
@@ -18,6 +20,8 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OUT = HERE / "libhqmq_amd.so"
+BENCH_SRC = HERE / "csrc_bench"
+BENCH_OUT = HERE / "libhqmq_bench.so"
 
 COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -53,13 +57,21 @@ def build(verbose: bool = False) -> Path:
             raise RuntimeError(f"hipcc failed on {src.name}")
         return obj
 
+    bench_srcs = sorted(BENCH_SRC.glob("*.hip"))
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
-        objs = list(ex.map(compile_one, srcs))
+        all_objs = list(ex.map(compile_one, srcs + bench_srcs))
+    objs, bench_objs = all_objs[:len(srcs)], all_objs[len(srcs):]
     cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode:
         sys.stderr.write(r.stdout + r.stderr)
         raise RuntimeError("link failed")
+    if bench_objs:
+        cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(BENCH_OUT), *map(str, bench_objs)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("link of the measurement library failed")
     return OUT
 
 

@@ -6,7 +6,7 @@
 
 #include "../../include/hqmq_amd.h"
 
-#define HQMQ_VERSION 0x000100
+#define HQMQ_VERSION 0x000200  // 0x000200: hqmq_packed gained scale_max_bits (every struct that embeds it moved), partial records are d_h + 4 floats, the read probes left the library
 
 namespace hqmq {
 

@@ -402,24 +402,3 @@ def attn_combine(partials: Optional[torch.Tensor], O: torch.Tensor, n_splits: in
                                           C.c_int(Tq), C.c_int(d_h), C.c_int(n_splits), L.i64(O.stride(0)), L.i64(O.stride(1)),
                                           L.i64(O.stride(2)), L.stream_ptr(O.device)), "hqmq_attn_combine")
     return O
-
-
-def read_ceiling(Kc, Vc, T_kv: int, *, H_q: int, n_splits: int = 0, depth: int = 3, waves: int = 8,
-                 kernel_events: Optional[tuple] = None) -> None:
-    """Measurement aid: launch the kernel that only reads the K and V planes with the decode-attention kernel's grid and
-    load pattern (hqmq_attn_read_ceiling); 16+0 layout at d_h 128 only."""
-    dev = Kc.device
-    a = L.AttnArgs()
-    a.K, a.V = Kc.c_struct(), Vc.c_struct()
-    a.dtype = L.DT_CODE[Kc.dtype]
-    a.B, a.H_q, a.H_kv, a.T_q, a.T_kv, a.n_chunks = Kc.B, H_q, Kc.H, 1, T_kv, Kc.n
-    a.t_cap = Kc.t_cap
-    a.idx_bits, a.main_bits, a.aux_bits, a.qmax = Kc.idx_bits, Kc.main_bits, Kc.aux_bits, Kc.qmax
-    a.n_splits = n_splits if n_splits > 0 else pick_splits(Kc.B, H_q, Kc.H, 1, T_kv)
-    if kernel_events is not None:
-        a.start_event, a.stop_event = C.c_void_p(kernel_events[0]), C.c_void_p(kernel_events[1])
-    nbytes = int(L.lib().hqmq_attn_read_ceiling_sink_bytes(C.c_int(Kc.B), C.c_int(Kc.H), C.c_int(a.n_splits)))
-    sink = _workspace(nbytes, dev, "ceiling")
-    with torch.cuda.device(dev):
-        L.check(L.lib().hqmq_attn_read_ceiling(C.byref(a), C.c_int(depth), C.c_int(waves), L.ptr(sink), L.i64(sink.numel()),
-                                               L.stream_ptr(dev)), "hqmq_attn_read_ceiling")

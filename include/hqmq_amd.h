@@ -220,7 +220,9 @@ typedef struct hqmq_attn_args {
     int n_splits;             /* 0 = choose */
     void *workspace; int64_t workspace_bytes;
     int skip_combine;         /* 1: leave the split partials in the workspace (merge later with hqmq_attn_combine) */
-    int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing) */
+    int force_generic;        /* 1: use the layout-generic kernel even where a specialised one exists (testing);
+                                 2: keep the specialised kernels that hold their tiles in registers where the kernel that
+                                 lands its loads in LDS would run (plain 16+0 caches at d_h 128; identical results) */
     const int32_t *kv_start;  /* [B] or NULL: first visible token of every sequence (left-padded batches) */
     const int32_t *batch_order; /* [B] or NULL: a permutation of 0..B-1, the order in which the sequences' blocks are
                                    started (pass the sequences sorted by length, longest first, for ragged batches) */
@@ -261,17 +263,6 @@ int hqmq_attn_combine(const void *workspace, void *O, int dtype, int B, int H_q,
 #define HQMQ_ATTN_STATIC_SCRATCH_BYTES (8 << 20)
 int64_t hqmq_attn_static_scratch_bytes(void);
 int hqmq_attn_fwd_static(const hqmq_attn_args *a, void *stream);
-
-/* Measurement aid, no counterpart in the reference: a kernel that only reads the K and V planes of a packed cache
- * with the grid, the per-wavefront token ranges and the per-lane loads of the specialised decode-attention kernel
- * (16+0 layout at d_h = 128, no sideband; other layouts return HQMQ_ERR_LAYOUT).  Its duration is the time the
- * memory system needs for a launch of this shape; bench.py reports it beside the attention kernel's.
- *   a       as for hqmq_attn_fwd (Q, O, tables and workspace are not touched; start_event / stop_event are honoured)
- *   depth   32-token steps per wavefront in the ring: depth - 1 are in flight (2, 3, 4 or 6; the attention kernel uses 3)
- *   waves   wavefronts per block, 8 or 12
- *   sink    hqmq_attn_read_ceiling_sink_bytes(B, H_kv, n_splits) bytes that receive one word per thread */
-int64_t hqmq_attn_read_ceiling_sink_bytes(int B, int H_kv, int n_splits);
-int hqmq_attn_read_ceiling(const hqmq_attn_args *a, int depth, int waves, void *sink, int64_t sink_bytes, void *stream);
 
 #ifdef __cplusplus
 }

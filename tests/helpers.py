@@ -161,3 +161,40 @@ def gpu_attention_refs(Qb, K_D, V_D, K_x, V_x):
     ref_d = attend(K_D, V_D)
     ref_x, a_abs = attend(K_x, V_x, V_x.abs())
     return ref_d, ref_x, a_abs
+
+
+def masked_two_refs(cache, Q, T, mask=None):
+    """The two fp32 references of assert_attention_close for a whole batch with an explicit visibility mask
+    (bool, broadcastable to (B, H_q, T_q, T); None = everything visible), computed on the cache's device from the
+    cache's own planes: attention over the D-rounded dense cache (what the reference attends over) and over the
+    unrounded product joint[idx] * (rq * rs / qmax) read by the independent bit reader (flagged chunks verbatim in
+    both).  Returns (ref_d, ref_x, attention-weighted |V|), each (B, H_q, T_q, d_h); softmax in float64; rows without a
+    visible token give 0."""
+    from hqmq_amd import ops
+    B, Hq, Tq, d = Q.shape
+    Hkv = cache.K.H
+    g = Hq // Hkv
+    K_D, V_D = ops.dequant_packed(cache.K, T, 0), ops.dequant_packed(cache.V, T, 0)
+    outs = ([], [], [])
+    for b in range(B):
+        K_x, V_x = exact_dense(cache.K, b, T, K_D[b]), exact_dense(cache.V, b, T, V_D[b])
+        q = Q[b].double().view(Hkv, g, Tq, d)
+        mb = None
+        if mask is not None:
+            mb = mask.expand(B, Hq, Tq, T)[b].view(Hkv, g, Tq, T)
+
+        def attend(K, V, Vabs=None):
+            s = torch.einsum("hgqd,hkd->hgqk", q, K.double()) * d ** -0.5
+            if mb is not None:
+                s = s.masked_fill(~mb, float("-inf"))
+            p = torch.nan_to_num(torch.softmax(s, dim=-1))
+            o = torch.einsum("hgqk,hkd->hgqd", p, V.double()).reshape(Hq, Tq, d).float()
+            if Vabs is None:
+                return o
+            return o, torch.einsum("hgqk,hkd->hgqd", p, Vabs.double()).reshape(Hq, Tq, d).float()
+
+        outs[0].append(attend(K_D[b], V_D[b]))
+        rx, ab = attend(K_x, V_x, V_x.abs())
+        outs[1].append(rx)
+        outs[2].append(ab)
+    return tuple(torch.stack(o).cpu() for o in outs)

@@ -148,7 +148,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in include/hqmq_amd.h but not exported"
     assert sorted(L.EXPORTS) == names
-    assert lib.hqmq_version() == 0x000100
+    assert lib.hqmq_version() == 0x000200
     assert lib.hqmq_status_string(-2).decode().startswith("a size")
 
 

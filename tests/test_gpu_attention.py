@@ -13,7 +13,7 @@ import torch
 from oracle import c_oracle as CO
 from oracle import torch_oracle as TO
 from tests.helpers import (DT, assert_attention_close, attention_refs, attn_tolerance, bit_equal, dense_from_codes,
-                           exact_dense, gpu_attention_refs, kv_input, unbits, unpack_planes)
+                           exact_dense, gpu_attention_refs, kv_input, masked_two_refs, unbits, unpack_planes)
 from tests.test_oracle import ATTN_CASES, load_attn_case
 
 pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a GPU")]
@@ -404,16 +404,12 @@ def test_clustered_outlier_channels(d_h, Tq, hot, dn):
     assert float(cache.K.sb_count.sum()) / (B * Hkv * T * d_h / 4) > 0.02
     Q = torch.randn(B, Hq, Tq, d_h, generator=g).to(dt).to(DEV)
     off = T - Tq
-    Kd = ops.dequant_packed(cache.K, T, 0).float().repeat_interleave(Hq // Hkv, 1)
-    Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
-    s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
     mask = torch.arange(T, device=DEV).view(1, 1, 1, T) <= (torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off)
-    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
-    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))     # bf16: the output's own rounding
+    refs = masked_two_refs(cache, Q, T, mask)
     for generic in (False, True):
         for ns in (0, 3):
             O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, force_generic=generic, n_splits=ns)
-            assert (O.float() - ref).abs().max().item() < tol, (generic, ns)
+            assert_attention_close(O, *refs, base=2e-3, what=f"generic={generic} n_splits={ns}")
 
 
 def _planted(B, H, T, d, seed, dt):
@@ -488,10 +484,11 @@ def test_crop_per_sequence_then_decode_appends():
     for bb in range(B):
         got = ops.dequant_packed(cache.K, Tm, 0)[bb, :, int(lens[bb]):int(lens[bb]) + 20].float()
         assert (got - k[bb, :, :20].float()).abs().mean().item() < 0.25 * k[bb, :, :20].float().abs().mean().item()
-    tol = 8e-3 * max(1.0, float(ref.abs().max()))
+    refs = masked_two_refs(cache, Q, Tm, mask)
     for generic in (False, True):
         O = hqmq.fused_attention_packed(Q, cache, causal=False, kv_lens=pos, T_kv=Tm, force_generic=generic)
-        assert (O.float() - ref).abs().max().item() < tol, generic
+        assert_attention_close(O, *refs, base=2e-3, what=f"generic={generic}")
+        assert (O.float() - ref).abs().max().item() < 2e-2 * max(1.0, float(ref.abs().max())), generic       # and the plain fp32 einsum, loosely
 
 
 @pytest.mark.parametrize("med3x,Tq", [(False, 1), (True, 1), (True, 24)])
@@ -575,11 +572,15 @@ def test_long_ranges_per_block(dn, kv_lens, S, b_r):
     if lens is not None:
         s = s.masked_fill(torch.arange(T, device=DEV).view(1, 1, 1, T) >= lens.view(B, 1, 1, 1), float("-inf"))
     ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
-    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))
+    vis = None if lens is None else torch.arange(T, device=DEV).view(1, 1, 1, T) < lens.view(B, 1, 1, 1)
+    refs = masked_two_refs(cache, Q, T, vis)
+    assert (refs[0].to(DEV) - ref).abs().max().item() < 1e-3 * max(1.0, float(ref.abs().max()))     # the helper against the plain einsum
     for ns in (1, 2):
         O = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns)
         Og = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns, force_generic=True)
-        assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
+        Or = hqmq.fused_attention_packed(Q, cache, kv_lens=lens, T_kv=T, n_splits=ns, force_generic=2)        # register-tile kernel
+        for name, o in (("specialised", O), ("generic", Og), ("register tiles", Or)):
+            assert_attention_close(o, *refs, base=2e-3, what=f"{name} n_splits={ns}")
 
 
 def test_long_ranges_per_block_outliers_d64():
@@ -599,11 +600,13 @@ def test_long_ranges_per_block_outliers_d64():
     Vd = ops.dequant_packed(cache.V, T, 0).float().repeat_interleave(Hq // Hkv, 1)
     s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
     ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, -1), Vd)
-    tol = 8e-3 * max(1.0, float(ref.abs().max()))
+    refs = masked_two_refs(cache, Q, T)
+    assert (refs[0].to(DEV) - ref).abs().max().item() < 1e-3 * max(1.0, float(ref.abs().max()))
     for ns in (1, 2):
         O = hqmq.fused_attention_packed(Q, cache, n_splits=ns)
         Og = hqmq.fused_attention_packed(Q, cache, n_splits=ns, force_generic=True)
-        assert (O.float() - ref).abs().max().item() < tol and (Og.float() - ref).abs().max().item() < tol, ns
+        assert_attention_close(O, *refs, base=2e-3, what=f"specialised n_splits={ns}")
+        assert_attention_close(Og, *refs, base=2e-3, what=f"generic n_splits={ns}")
 
 
 @pytest.mark.parametrize("S,b_r,dn,d_h", [(96, 4, "fp16", 128), (24, 3, "bf16", 128), (192, 6, "fp16", 128), (96, 4, "bf16", 64)])
@@ -627,12 +630,13 @@ def test_prefill_two_column_groups(S, b_r, dn, d_h):
     s = torch.einsum("bhqd,bhkd->bhqk", Q.float(), Kd) * d_h ** -0.5
     mask = torch.arange(T, device=DEV).view(1, 1, 1, T) <= (torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off)
     ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s.masked_fill(~mask, float("-inf")), -1), Vd)
-    tol = (2e-3 if dn == "fp16" else 8e-3) * max(1.0, float(ref.abs().max()))
+    refs = masked_two_refs(cache, Q, T, mask)
+    assert (refs[0].to(DEV) - ref).abs().max().item() < 1e-3 * max(1.0, float(ref.abs().max()))
     for ns in (2, 4):                       # 2 splits x 38 pairs of column groups x 4 (b, h) = 304 blocks
         O = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=ns)
-        assert (O.float() - ref).abs().max().item() < tol, ns
+        assert_attention_close(O, *refs, base=2e-3, what=f"n_splits={ns}")
     Og = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=2, force_generic=True)
-    assert (Og.float() - ref).abs().max().item() < tol
+    assert_attention_close(Og, *refs, base=2e-3, what="generic")
     # the same with per-sequence limits on both sides (left padding and a shorter second sequence)
     starts = torch.tensor([0, 70], dtype=torch.int32, device=DEV)
     lens = torch.tensor([T, 650], dtype=torch.int32, device=DEV)
@@ -640,4 +644,43 @@ def test_prefill_two_column_groups(S, b_r, dn, d_h):
     mask2 = mask & (kk >= starts.view(B, 1, 1, 1)) & (kk < lens.view(B, 1, 1, 1))
     ref2 = torch.einsum("bhqk,bhkd->bhqd", torch.nan_to_num(torch.softmax(s.masked_fill(~mask2, float("-inf")), -1)), Vd)
     O2 = hqmq.fused_attention_packed(Q, cache, causal=True, causal_offset=off, n_splits=2, kv_starts=starts, kv_lens=lens, T_kv=T)
-    assert (O2.float() - ref2).abs().max().item() < tol
+    refs2 = masked_two_refs(cache, Q, T, mask2)
+    assert (refs2[0].to(DEV) - ref2).abs().max().item() < 1e-3 * max(1.0, float(ref2.abs().max()))
+    assert_attention_close(O2, *refs2, base=2e-3, what="left padding and a shorter sequence")
+
+
+@pytest.mark.parametrize("dn,T,B,Tq,causal,ns,lens", [
+    ("fp16", 32, 1, 1, False, 0, None), ("fp16", 96, 1, 1, False, 0, None), ("fp16", 1000, 1, 1, False, 0, None),
+    ("fp16", 8192, 1, 1, False, 0, None), ("fp16", 777, 3, 1, False, 2, None), ("fp16", 5000, 2, 1, False, 0, [4100, 37]),
+    ("fp16", 2048, 1, 3, True, 0, None), ("bf16", 4096, 1, 1, False, 0, None), ("bf16", 20000, 2, 1, False, 3, None),
+    ("bf16", 300, 1, 4, True, 0, None), ("fp16", 33, 1, 1, False, 1, None), ("fp16", 3000, 2, 1, False, 5, [0, 2999])])
+def test_lds_landing_kernel_equals_register_tile_kernel(dn, T, B, Tq, causal, ns, lens):
+    """Plain s96_r4 caches at d_h 128 take the kernel whose loads land in LDS (tables, query rows and planes through
+    global_load_lds, hand-written waits).  It performs the arithmetic of the register-tile kernel in the same order, so
+    the two must agree bit for bit (force_generic=2 selects the register-tile kernel); both are held to the
+    two-reference bound, and so is the layout-generic kernel."""
+    import hqmq
+    dt = DT[dn]
+    Hq, Hkv, d_h = 8, 2, 128
+    g = torch.Generator().manual_seed(T + 7 * B)
+    k, v = torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV), torch.randn(B, Hkv, T, d_h, generator=g).to(dt).to(DEV)
+    q = hqmq.HQMQ(n_layers=2, n_heads=Hkv, secondary_size=96, radius_bits=4, device=DEV)
+    cache = q.new_cache(B, T, d_h, dt, layer_idx=1)
+    q.append(cache, k, v, 1)
+    Q = torch.randn(B, Hq, Tq, d_h, generator=g).to(dt).to(DEV)
+    kv_lens = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    off = T - Tq
+    kw = dict(causal=causal, causal_offset=off if causal else 0, n_splits=ns, kv_lens=kv_lens, T_kv=T)
+    O = hqmq.fused_attention_packed(Q, cache, **kw)
+    Or = hqmq.fused_attention_packed(Q, cache, force_generic=2, **kw)
+    Og = hqmq.fused_attention_packed(Q, cache, force_generic=True, **kw)
+    assert torch.equal(O, Or)
+    kk = torch.arange(T, device=DEV).view(1, 1, 1, T)
+    mask = torch.ones(B, 1, Tq, T, dtype=torch.bool, device=DEV)
+    if causal:
+        mask = mask & (kk <= torch.arange(Tq, device=DEV).view(1, 1, Tq, 1) + off)
+    if kv_lens is not None:
+        mask = mask & (kk < kv_lens.view(B, 1, 1, 1))
+    refs = masked_two_refs(cache, Q, T, mask)
+    assert_attention_close(O, *refs, base=2e-3, what="LDS landing")
+    assert_attention_close(Og, *refs, base=2e-3, what="generic")
