@@ -223,7 +223,7 @@ def gpu_config1(dev, calls=10):
     cache = fresh[-1]
     cache.K.check_overflow()
     cache.V.check_overflow()
-    Kd, Vd = ops.dequant_packed(cache.K, T, 0), ops.dequant_packed(cache.V, T, 0)
+    Kd, Vd = ops.dequant_packed(cache.K, T, 1), ops.dequant_packed(cache.V, T, 1)       # the quantizer's own rounding: the reference's output tensor
     chunks = 8 * T * d // 4
     return {"what": "BASELINE config 1 on the GPU: one bulk append = quantize (s24_r3) + Med3x (C = 3) + bit-packing + sideband of K and V, "
                     "8 heads x 2048 tokens x d_h 128 fp16; MSE of the cache dequantized again (packed codes + verbatim outlier chunks) "
@@ -455,6 +455,7 @@ def main():
         slice_bytes = cache_bytes * slice_tokens / T
         qsec, qtok, qmse = cpu_quantize_baseline_config1()
         if "config1" in result:
+            result["config1"]["mse_equal_to_cpu"] = bool(result["config1"]["mse_K"] == qmse[0] and result["config1"]["mse_V"] == qmse[1])
             result["config1"].update(cpu_us_per_call_K_and_V=round(qsec * 1e6, 1), cpu_GTok_per_s=round(qtok / qsec / 1e9, 8),
                                      cpu_mse_K=qmse[0], cpu_mse_V=qmse[1], cpu_cores=threads,
                                      cpu_what="the restated reference quantizer (oracle, torch on the host) on the same tensors")

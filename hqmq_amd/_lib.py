@@ -71,6 +71,12 @@ class AttnArgs(C.Structure):
     ]
 
 
+class PackedRows(C.Structure):
+    """hqmq_packed_rows: the packed planes of the rows a compaction call covers."""
+    _fields_ = [("main_plane", vp), ("aux_plane", vp), ("scale_plane", vp),
+                ("idx_bits", C.c_int), ("main_bits", C.c_int), ("aux_bits", C.c_int), ("qmax", C.c_int)]
+
+
 EXPORTS = [
     "hqmq_version", "hqmq_status_string", "hqmq_layout_bits", "hqmq_build_joint", "hqmq_quantize",
     "hqmq_med3x_workspace_bytes", "hqmq_med3x_threshold", "hqmq_outlier_mask", "hqmq_outlier_compact", "hqmq_dequant",

@@ -22,7 +22,10 @@ extern "C" int hqmq_append_kv(const hqmq_append_args *k, const hqmq_append_args 
                                a[i]->median, a[i]->thr, a[i]->n_out};
         cmp[n_med] = CompactCall{q[i].x, q[i].x_stride_b, q[i].x_stride_h, q[i].x_stride_t, q[i].dtype, q[i].B, q[i].H, q[i].T,
                                  q[i].n_chunks, q[i].flag_plane, q[i].t_cap, q[i].t_off, q[i].pos, a[i]->sideband,
-                                 a[i]->sb_cap, a[i]->sb_tile_off, a[i]->sb_count, a[i]->overflow, a[i]->sb_coord};
+                                 a[i]->sb_cap, a[i]->sb_tile_off, a[i]->sb_count, a[i]->overflow, a[i]->sb_coord,
+                                 q[i].main_plane, q[i].aux_plane, q[i].scale_plane, 0, q[i].main_bits, q[i].aux_bits,
+                                 (1 << q[i].radius_bits) - 1};
+        if (layout_bits(q[i].secondary_size, q[i].radius_bits, &cmp[n_med].idx_bits, nullptr, nullptr)) return HQMQ_ERR_SHAPE;
         const int rc = check_compact(cmp[n_med]);
         if (rc) return rc;
         with_q[i] = &cmp[n_med];

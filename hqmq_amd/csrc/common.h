@@ -101,7 +101,48 @@ struct CompactCall {
     int dtype, B, H, T, n;
     const uint8_t *flag_plane; int64_t t_cap; int t_off; const int32_t *pos;
     void *sideband; int64_t sb_cap; int32_t *sb_tile_off, *sb_count, *overflow; uint16_t *sb_coord;
+    // the packed planes of the same rows (main_plane NULL: none).  With them a flagged chunk that finds the sideband
+    // full is turned back into a plain chunk (flag bit cleared, its radius code written) instead of decoding to zero.
+    uint8_t *main_plane, *aux_plane; const void *scale_plane; int idx_bits, main_bits, aux_bits, qmax;
 };
+
+// ORs `width` bits of `val` into a little-endian bit stream at bit `pos` of `row` (the field holds zeros); other
+// threads may do the same to neighbouring fields of the same bytes.
+__device__ __forceinline__ void or_bit_field(uint8_t *row, int pos, uint32_t val, int width) {
+    if (width <= 0 || val == 0u) return;
+    const uint64_t v = (uint64_t)(val & ((1u << width) - 1u)) << (pos & 7);
+    uint8_t *p = row + (pos >> 3);
+    for (int i = 0; i * 8 < (pos & 7) + width; i++) {
+        const uint32_t byte = (uint32_t)(v >> (8 * i)) & 0xffu;
+        if (!byte) continue;
+        const uintptr_t a = (uintptr_t)(p + i);
+        atomicOr(reinterpret_cast<uint32_t *>(a & ~(uintptr_t)3), byte << (8 * (a & 3)));
+    }
+}
+
+// A flagged chunk for which the sideband has no room left degrades to a plain HQMQ chunk: its flag bit is cleared and
+// the radius code that the quantizer would have stored for an unflagged chunk is written into its (zero) radius field
+// (the reference never loses an outlier, src/quantizers/outlier_aware.py:86; a full sideband costs accuracy here, not
+// the chunk).  xc: the chunk's four input values; prow: the row's index in the [B][H][t_cap] planes.
+// Built with -ffp-contract=off like the quantizer: the same roundings, the same code.
+template <class D>
+__device__ __forceinline__ void degrade_to_plain(const CompactCall &a, size_t prow, int c, const typename D::storage *xc) {
+    if (!a.main_plane || !a.scale_plane) return;
+    const float nrm = D::rnd(norm4(D::load(xc), D::load(xc + 1), D::load(xc + 2), D::load(xc + 3)));
+    const float r = clamp_min_d<D>(nrm, 1e-8f);
+    const float rm = D::load((const typename D::storage *)a.scale_plane + prow);
+    const float qmaxf = (float)a.qmax;
+    const float scale = D::rnd(rm / qmaxf);
+    float qf = rintf(D::rnd(r / scale));
+    if (!is_nan(qf)) qf = fminf(fmaxf(qf, 0.f), qmaxf);
+    const uint32_t rq = is_nan(qf) ? 0u : (uint32_t)(int)qf;
+    const int in_main = a.main_bits - a.idx_bits;                  // radius bits that live in the main field
+    if (in_main > 0) or_bit_field(a.main_plane + prow * (size_t)((a.n * a.main_bits + 7) >> 3), c * a.main_bits + a.idx_bits, rq, in_main);
+    if (a.aux_plane && a.aux_bits > 0)
+        or_bit_field(a.aux_plane + prow * (size_t)((a.n * a.aux_bits + 7) >> 3), c * a.aux_bits, in_main > 0 ? rq >> in_main : rq, a.aux_bits);
+    const uintptr_t fa = (uintptr_t)(const_cast<uint8_t *>(a.flag_plane) + prow * (size_t)((a.n + 7) >> 3) + (c >> 3));
+    atomicAnd(reinterpret_cast<uint32_t *>(fa & ~(uintptr_t)3), ~((1u << (c & 7)) << (8 * (fa & 3))));
+}
 int med3x_calls(const Med3xCall *c, int count, hipStream_t st);                                            // med3x.hip
 int compact_calls(const CompactCall *c, int count, hipStream_t st);                                        // med3x.hip
 int check_compact(const CompactCall &c);                                                                   // med3x.hip

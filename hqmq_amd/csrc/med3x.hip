@@ -410,13 +410,18 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
             if ((row & (kTile - 1)) == 0) sb_tile_off[(size_t)bh * tiles + (row >> 4)] = before;
             int k = before;
             const ST *xr = x + b * xsb + h * xsh + (int64_t)t * xst;
+            uint8_t own[32];                                       // the row's flags as they were (bits may be cleared below)
+            for (int by = 0; by < frb && by < 32; by++) own[by] = fr[by];
             for (int c = 0; c < n && cnt; c++) {
-                if ((fr[c >> 3] >> (c & 7)) & 1) {
+                if ((own[c >> 3] >> (c & 7)) & 1) {
                     if (k < sb_cap) {
                         ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                         for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
                         if (sb_coord) sb_coord[(size_t)bh * sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
-                    } else *overflow = 1;
+                    } else {
+                        *overflow = 1;
+                        degrade_to_plain<D>(a, (size_t)bh * t_cap + row, c, xr + c * 4);
+                    }
                     k++;
                 }
             }
@@ -480,11 +485,17 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(int64_t t_cap, int row0
     if (threadIdx.x == 1023) sb_count[bh] = base + part[1023];
 }
 // Pass 3: one thread per new row copies the row's flagged chunks behind those of the tile's earlier rows.
+// (A row whose entries do not fit clears flag bits while its neighbours count them: every entry they then fail to
+// count lay beyond the capacity, so their own entries still come out beyond it, and the offsets of the entries that
+// fit do not move.)
 template <class D>
-__global__ void tile_copy_kernel(const typename D::storage *x, int64_t xsb, int64_t xsh, int64_t xst, int H, int T, int n,
-                                 const uint8_t *flag_plane, int64_t t_cap, int row0, typename D::storage *sideband, int64_t sb_cap,
-                                 const int32_t *sb_tile_off, int32_t *overflow, uint16_t *sb_coord) {
+__global__ void tile_copy_kernel(CompactCall a) {
     using ST = typename D::storage;
+    const ST *x = (const ST *)a.x;
+    ST *sideband = (ST *)a.sideband;
+    const int H = a.H, T = a.T, n = a.n, row0 = a.t_off;
+    const int64_t t_cap = a.t_cap, sb_cap = a.sb_cap;
+    const uint8_t *flag_plane = a.flag_plane;
     const int bh = blockIdx.y, b = bh / H, h = bh - b * H;
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= T) return;
@@ -492,21 +503,25 @@ __global__ void tile_copy_kernel(const typename D::storage *x, int64_t xsb, int6
     const int64_t tiles = (t_cap + kTile - 1) / kTile;
     const int row = row0 + t, tile_row = row & ~(kTile - 1);
     const uint8_t *fr = flag_plane + ((size_t)bh * t_cap + row) * frb;
+    uint8_t mine[32];
     int own = 0;
-    for (int k = 0; k < frb; k++) own += __popc((uint32_t)fr[k]);
+    for (int k = 0; k < frb && k < 32; k++) { mine[k] = fr[k]; own += __popc((uint32_t)mine[k]); }
     if (!own) return;
-    int before = sb_tile_off[(size_t)bh * tiles + (row >> 4)];
+    int before = a.sb_tile_off[(size_t)bh * tiles + (row >> 4)];
     const uint8_t *f0 = flag_plane + ((size_t)bh * t_cap + tile_row) * frb;
     for (int k = 0; k < (row - tile_row) * frb; k++) before += __popc((uint32_t)f0[k]);
-    const ST *xr = x + b * xsb + h * xsh + (int64_t)t * xst;
+    const ST *xr = x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst;
     int k = before;
     for (int c = 0; c < n; c++) {
-        if ((fr[c >> 3] >> (c & 7)) & 1) {
+        if ((mine[c >> 3] >> (c & 7)) & 1) {
             if (k < sb_cap) {
                 ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                 for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
-                if (sb_coord) sb_coord[(size_t)bh * sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
-            } else *overflow = 1;
+                if (a.sb_coord) a.sb_coord[(size_t)bh * sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
+            } else {
+                *a.overflow = 1;
+                degrade_to_plain<D>(a, (size_t)bh * t_cap + row, c, xr + c * 4);
+            }
             k++;
         }
     }
@@ -627,13 +642,11 @@ static int compact_one(const CompactCall &c, hipStream_t st) {
                            c.T, frb, n_tiles, c.sb_tile_off);
         hipLaunchKernelGGL(tile_scan_kernel, dim3(c.B * c.H), dim3(1024), 0, st, c.t_cap, c.t_off, n_tiles, c.sb_tile_off, c.sb_count);
         dim3 cgrid((c.T + 255) / 256, c.B * c.H);
-#define COPY(DT, ST)                                                                                                       \
-    hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, (const ST *)c.x, c.xsb, c.xsh, c.xst, c.H, c.T, c.n,     \
-                       c.flag_plane, c.t_cap, c.t_off, (ST *)c.sideband, c.sb_cap, c.sb_tile_off, c.overflow, c.sb_coord)
+#define COPY(DT) hipLaunchKernelGGL(tile_copy_kernel<DT>, cgrid, dim3(256), 0, st, c)
         switch (c.dtype) {
-            case HQMQ_F32: COPY(F32, float); break;
-            case HQMQ_F16: COPY(F16, uint16_t); break;
-            default: COPY(BF16, uint16_t); break;
+            case HQMQ_F32: COPY(F32); break;
+            case HQMQ_F16: COPY(F16); break;
+            default: COPY(BF16); break;
         }
 #undef COPY
         return hip_status(hipGetLastError());
@@ -676,11 +689,20 @@ int hqmq::compact_calls(const CompactCall *c, int count, hipStream_t st) {
 }
 
 extern "C" int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype, int B,
-                                    int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
+                                    int H, int T, int n_chunks, uint8_t *flag_plane, int64_t t_cap, int t_off,
                                     const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off,
-                                    int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord, void *stream) {
-    const CompactCall c{x, x_stride_b, x_stride_h, x_stride_t, dtype, B, H, T, n_chunks, flag_plane, t_cap, t_off, pos,
-                        sideband, sb_cap, sb_tile_off, sb_count, overflow, sb_coord};
+                                    int32_t *sb_count, int32_t *overflow, uint16_t *sb_coord, const hqmq_packed_rows *planes,
+                                    void *stream) {
+    CompactCall c{x, x_stride_b, x_stride_h, x_stride_t, dtype, B, H, T, n_chunks, flag_plane, t_cap, t_off, pos,
+                  sideband, sb_cap, sb_tile_off, sb_count, overflow, sb_coord, nullptr, nullptr, nullptr, 0, 0, 0, 0};
+    if (planes) {
+        if (!planes->main_plane || !planes->scale_plane || (planes->aux_bits > 0 && !planes->aux_plane)) return HQMQ_ERR_NULL;
+        if (planes->idx_bits < 1 || planes->main_bits < planes->idx_bits - 8 || planes->main_bits > 16 || planes->aux_bits < 0 ||
+            planes->aux_bits > 8 || planes->qmax < 1)
+            return HQMQ_ERR_LAYOUT;
+        c.main_plane = planes->main_plane; c.aux_plane = planes->aux_plane; c.scale_plane = planes->scale_plane;
+        c.idx_bits = planes->idx_bits; c.main_bits = planes->main_bits; c.aux_bits = planes->aux_bits; c.qmax = planes->qmax;
+    }
     return compact_calls(&c, 1, (hipStream_t)stream);
 }
 

@@ -479,18 +479,53 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
 
     // ---- packed rows ----
     if (a.main_plane || a.flag_plane || a.scale_plane) {
-        // a flagged chunk is read from the sideband; its packed code keeps idx with radius code 0, which decodes to zero
-        code_sh[tid] = (uint32_t)idx | ((uint32_t)(flagged ? 0 : rq) << a.idx_bits);
-        mask_sh[tid] = flagged ? 1u : 0u;
-        __syncthreads();
         const int64_t row = (a.pos ? a.pos[b] : 0) + a.t_off + t;
         const bool row_ok = active && writer && row >= 0 && row < a.t_cap;  // a bad pos[] must not write outside the plane
+        // Sideband compaction in the same launch, for appends whose new rows of a (b, h) all sit in this block
+        // (T <= tokens_per_block; n a power of two, so the lanes of a token share a wavefront).  Entries, tile
+        // offsets and counters come out as the in-order compaction kernel leaves them: flagged chunks in
+        // (row, chunk) order behind the entries already there, the offset of a tile = the count before its
+        // first row.  The entry slots are worked out before the rows are packed: a flagged chunk that finds the
+        // sideband full is packed as a plain chunk (its radius code, no flag) instead of decoding to zero.
+        bool keep = flagged;            // stays an outlier in the packed planes
+        bool entry = false;             // this lane writes a sideband entry
+        int ent_slot = 0, tile_first = 0, ent_total = 0;
+        if (a.compact) {
+            __syncthreads();            // radius_sh is free from here on
+            const bool f = row_ok && flagged;
+            const uint64_t m = __builtin_amdgcn_ballot_w64(f);
+            const int lane = tid & 63;
+            const uint64_t tok_bits = n == 64 ? ~0ull : ((1ull << n) - 1ull) << ((lane / n) * n);
+            const int before_c = __popcll(m & tok_bits & ((1ull << lane) - 1ull));
+            int *cnt_sh = reinterpret_cast<int *>(radius_sh);           // free since the scales were taken
+            if (c == 0 && tok_local < a.tokens_per_block) cnt_sh[tok_local] = __popcll(m & tok_bits);
+            const int base = a.sb_count[(size_t)b * a.H + h];           // read by every thread before the barrier,
+            __syncthreads();                                            // rewritten by one thread at the end
+            int mine = base, total = base;
+            for (int i = 0; i < a.T; i++) {
+                const int ci = cnt_sh[i];
+                if (i < tok_local) mine += ci;
+                total += ci;
+            }
+            tile_first = mine;
+            ent_total = total;
+            ent_slot = mine + before_c;
+            entry = f && ent_slot < a.sb_cap;
+            if (f && !entry) {
+                keep = false;
+                *a.overflow = 1;
+            }
+        }
+        // a flagged chunk is read from the sideband; its packed code keeps idx with radius code 0, which decodes to zero
+        code_sh[tid] = (uint32_t)idx | ((uint32_t)(keep ? 0 : rq) << a.idx_bits);
+        mask_sh[tid] = keep ? 1u : 0u;
+        __syncthreads();
         // one-bit planes (flags, a one-bit aux field) of tokens whose lanes sit side by side in a wavefront come
         // straight from a ballot: the token's n bits are n / 8 whole bytes of it
         const bool side_by_side = (n & (n - 1)) == 0 && n >= 8 && n <= 64;
         const int lane_base = (tid & 63) / n * n;
         const uint64_t aux_bits1 = __builtin_amdgcn_ballot_w64(((code_sh[tid] >> a.main_bits) & 1u) != 0u);
-        const uint64_t flag_bits1 = __builtin_amdgcn_ballot_w64(flagged);
+        const uint64_t flag_bits1 = __builtin_amdgcn_ballot_w64(keep);
         if (row_ok) {
             const size_t prow = ((size_t)b * a.H + h) * a.t_cap + row;
             const uint32_t *codes = code_sh + tok_local * n;
@@ -540,43 +575,18 @@ __device__ __forceinline__ void quantize_body(const QParams &a) {
                 atomicMax(a.scale_max, mine);
         }
         if (a.compact) {
-            // Sideband compaction in the same launch, for appends whose new rows of a (b, h) all sit in this block
-            // (T <= tokens_per_block; n a power of two, so the lanes of a token share a wavefront).  Entries, tile
-            // offsets and counters come out as the in-order compaction kernel leaves them: flagged chunks in
-            // (row, chunk) order behind the entries already there, the offset of a tile = the count before its
-            // first row.
-            const bool f = row_ok && flagged;
-            const uint64_t m = __builtin_amdgcn_ballot_w64(f);
-            const int lane = tid & 63;
-            const uint64_t tok_bits = n == 64 ? ~0ull : ((1ull << n) - 1ull) << ((lane / n) * n);
-            const int before_c = __popcll(m & tok_bits & ((1ull << lane) - 1ull));
-            int *cnt_sh = reinterpret_cast<int *>(radius_sh);           // free since the scales were taken
-            if (c == 0 && tok_local < a.tokens_per_block) cnt_sh[tok_local] = __popcll(m & tok_bits);
             const size_t bhs = (size_t)b * a.H + h;
-            const int base = a.sb_count[bhs];                           // read by every thread before the barrier,
-            __syncthreads();                                            // rewritten by one thread after it
-            int mine = base, total = base;
-            for (int i = 0; i < a.T; i++) {
-                const int ci = cnt_sh[i];
-                if (i < tok_local) mine += ci;
-                total += ci;
-            }
             if (row_ok) {
                 const int64_t tiles = (a.t_cap + kTile - 1) / kTile;
-                if (c == 0 && (row & (kTile - 1)) == 0) a.sb_tile_off[bhs * tiles + (row >> 4)] = mine;
-                if (f) {
-                    const int k = mine + before_c;
-                    if (k < a.sb_cap) {
-                        const ST *xp = (const ST *)a.x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst + c * 4;
-                        ST *dst = (ST *)a.sideband + (bhs * a.sb_cap + k) * 4;
-                        for (int j = 0; j < 4; j++) dst[j] = xp[j];
-                        if (a.sb_coord) a.sb_coord[bhs * a.sb_cap + k] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
-                    } else {
-                        *a.overflow = 1;
-                    }
+                if (c == 0 && (row & (kTile - 1)) == 0) a.sb_tile_off[bhs * tiles + (row >> 4)] = tile_first;
+                if (entry) {
+                    const ST *xp = (const ST *)a.x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst + c * 4;
+                    ST *dst = (ST *)a.sideband + (bhs * a.sb_cap + ent_slot) * 4;
+                    for (int j = 0; j < 4; j++) dst[j] = xp[j];
+                    if (a.sb_coord) a.sb_coord[bhs * a.sb_cap + ent_slot] = (uint16_t)(((row & (kTile - 1)) << 8) | c);
                 }
             }
-            if (tid == 0) a.sb_count[bhs] = total;
+            if (tid == 0) a.sb_count[bhs] = ent_total;
         }
     }
 }

@@ -21,6 +21,8 @@ from __future__ import annotations
 
 from typing import Optional
 
+import warnings
+
 import torch
 from transformers import AttentionInterface, DynamicCache
 from transformers.cache_utils import DynamicLayer
@@ -53,11 +55,13 @@ class PackedLayer(DynamicLayer):
         self.quantizer, self.layer_idx, self.max_tokens, self.sideband_frac = quantizer, layer_idx, max_tokens, sideband_frac
         self.packed = None
         self.n_tokens = 0
-        # a sideband that runs full drops outlier chunks (they then decode to zero): the flag the kernels set is read
-        # back after the first append (the prefill) and then once every `overflow_check_every` appends (one device
-        # read each time; 0 = never, call check_overflow() yourself)
+        # a sideband that runs full stores further outlier chunks as plain HQMQ chunks: the flag the kernels set is
+        # read back after the first append (the prefill) and then once every `overflow_check_every` appends (one
+        # device read for K and V together, never under stream capture; 0 = never, call check_overflow() yourself),
+        # and a warning is issued once
         self.overflow_check_every = overflow_check_every
         self._appends = 0
+        self._warned = False
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, *args, **kwargs):
         if self.packed is None:
@@ -72,10 +76,12 @@ class PackedLayer(DynamicLayer):
         self.quantizer.append(self.packed, key_states, value_states, self.layer_idx)
         self.n_tokens += key_states.shape[2]
         self._appends += 1
-        if self.packed.K.has_outliers and self.overflow_check_every and (
-                self._appends == 1 or self._appends % self.overflow_check_every == 0):
-            self.packed.K.check_overflow()
-            self.packed.V.check_overflow()
+        if self.packed.K.has_outliers and self.overflow_check_every and not self._warned and (
+                self._appends == 1 or self._appends % self.overflow_check_every == 0) and not torch.cuda.is_current_stream_capturing():
+            if int((self.packed.K.sb_overflow | self.packed.V.sb_overflow).item()):          # K and V in one read
+                self._warned = True
+                warnings.warn(f"layer {self.layer_idx}: the outlier sideband is full; further outlier chunks are stored as plain "
+                              f"HQMQ chunks (accuracy of those chunks, not data, is lost). Raise sideband_frac ({self.sideband_frac}).")
         key_states.hqmq_layer = self          # how hqmq_packed_attention finds the planes
         return key_states, value_states
 

@@ -176,12 +176,15 @@ def outlier_compact(x: torch.Tensor, cache, t_off: int = 0, pos: Optional[torch.
     dev = x.device
     if pos is not None:
         pos = pos.to(device=dev, dtype=torch.int32).contiguous()
+    rows = L.PackedRows()      # the planes of the same rows: a chunk that finds the sideband full goes back to a plain chunk
+    rows.main_plane, rows.aux_plane, rows.scale_plane = L.ptr(cache.main), L.ptr(cache.aux), L.ptr(cache.scale)
+    rows.idx_bits, rows.main_bits, rows.aux_bits, rows.qmax = cache.idx_bits, cache.main_bits, cache.aux_bits, cache.qmax
     with torch.cuda.device(dev):
         L.check(L.lib().hqmq_outlier_compact(
             L.ptr(x), L.i64(x.stride(0)), L.i64(x.stride(1)), L.i64(x.stride(2)), C.c_int(_dt(x)), C.c_int(B), C.c_int(H),
             C.c_int(T), C.c_int(d_h // 4), L.ptr(cache.flags), L.i64(cache.t_cap), C.c_int(t_off), L.ptr(pos),
             L.ptr(cache.sideband), L.i64(cache.sb_cap), L.ptr(cache.sb_tile_off), L.ptr(cache.sb_count),
-            L.ptr(cache.sb_overflow), L.ptr(cache.sb_coord), L.stream_ptr(dev)), "hqmq_outlier_compact")
+            L.ptr(cache.sb_overflow), L.ptr(cache.sb_coord), C.byref(rows), L.stream_ptr(dev)), "hqmq_outlier_compact")
 
 
 def append_kv(k: torch.Tensor, v: torch.Tensor, k_cache, v_cache, k_joint, k_slack, v_joint, v_slack, radius_bits: int, *,

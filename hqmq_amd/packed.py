@@ -99,7 +99,9 @@ class PackedTensor:
         s.scale_max_bits = L.ptr(self.scale_max)
         return s
 
-    RANGE_CHECK_EVERY = 256
+    RANGE_CHECK_EVERY = 256     # small appends between two reads of the largest scale; set it to 1 (per cache or on the
+                                # class) to read after every append: one device read each, and no window in which a bf16
+                                # scale that left [2^-8, 2^15) still meets the unguarded kernels
 
     def refresh_range(self) -> bool:
         """Reads the largest scale written so far (one device read) and records whether it lies outside [2^-8, 2^15),
@@ -168,11 +170,18 @@ class PackedTensor:
         view.wide_range, view._huge = self.wide_range, self._huge
         return view
 
+    def overflowed(self) -> bool:
+        """True if an append found the sideband full (reads one int from the device).  The chunks that found no room
+        were kept as plain HQMQ chunks (flag cleared, radius code written): nothing decodes to zero, the price is the
+        accuracy of those chunks."""
+        return self.sb_overflow is not None and bool(int(self.sb_overflow.item()))
+
     def check_overflow(self) -> None:
-        """Raises if an append ran out of sideband room (reads one int from the device)."""
-        if self.sb_overflow is not None and int(self.sb_overflow.item()):
-            raise L.HqmqError(f"outlier sideband overflow: more than {self.sb_cap} flagged chunks in one (b, h) stream; "
-                              "allocate the cache with a larger sideband_frac")
+        """Raises if an append ran out of sideband room (see overflowed)."""
+        if self.overflowed():
+            raise L.HqmqError(f"outlier sideband overflow: more than {self.sb_cap} flagged chunks in one (b, h) stream "
+                              "(the chunks beyond it were stored as plain HQMQ chunks); allocate the cache with a larger "
+                              "sideband_frac")
 
 
 @dataclass

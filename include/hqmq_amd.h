@@ -127,11 +127,22 @@ int hqmq_outlier_mask(const void *x, int64_t x_stride_b, int64_t x_stride_h, int
  * count them twice.  To rewrite rows, reset sb_count and the tile offsets to the state before them.)
  * sb_coord [B][H][sb_cap] (may be NULL): (row & 15) << 8 | chunk of every sideband entry, which lets the
  * specialised attention kernels walk the sideband densely; sb_tile_off must start out as INT32_MAX (tiles not
- * yet written read as "no entries"). */
+ * yet written read as "no entries").
+ * A full sideband: *overflow is set to 1, and with `planes` (the packed planes that hqmq_quantize wrote for the
+ * same rows) every flagged chunk that finds no room is turned back into a plain chunk: its flag bit is cleared and
+ * the radius code the quantizer gives an unflagged chunk is written into its radius field, so that it decodes as
+ * plain HQMQ instead of zero (the reference never loses an outlier, src/quantizers/outlier_aware.py:86; here a full
+ * sideband costs accuracy, never the chunk).  Without `planes` (NULL) such chunks keep radius code 0 and decode to
+ * zero: check *overflow.  hqmq_append_kv always passes the planes. */
+typedef struct hqmq_packed_rows {
+    uint8_t *main_plane, *aux_plane;  /* as passed to hqmq_quantize (aux_plane NULL when aux_bits = 0) */
+    const void *scale_plane;          /* D, [B][H][t_cap] */
+    int idx_bits, main_bits, aux_bits, qmax;
+} hqmq_packed_rows;
 int hqmq_outlier_compact(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int dtype,
-                         int B, int H, int T, int n_chunks, const uint8_t *flag_plane, int64_t t_cap, int t_off,
+                         int B, int H, int T, int n_chunks, uint8_t *flag_plane, int64_t t_cap, int t_off,
                          const int32_t *pos, void *sideband, int64_t sb_cap, int32_t *sb_tile_off, int32_t *sb_count,
-                         int32_t *overflow, uint16_t *sb_coord, void *stream);
+                         int32_t *overflow, uint16_t *sb_coord, const hqmq_packed_rows *planes, void *stream);
 
 /* One append of new K and V rows to a packed cache: Med3x threshold (when median_mult > 0), quantize + pack,
  * sideband compaction, for both tensors.  The results are those of hqmq_med3x_threshold, hqmq_quantize and

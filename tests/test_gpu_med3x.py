@@ -229,3 +229,62 @@ def test_full_size_median_properties():
         slack = N // 1000                                        # torch's norm may round a few values the other way
         assert int((nh < med[h]).sum()) <= N // 2 + slack and int((nh > med[h]).sum()) <= N // 2 + slack
     assert 0.01 < float(cnt.sum()) / norms.numel() < 0.04
+
+
+@pytest.mark.parametrize("dn,S,b_r,T,p,single", [("fp16", 96, 4, 600, 0.06, False), ("bf16", 24, 3, 600, 0.06, False), ("fp16", 192, 6, 100, 0.1, False),
+                                                 ("bf16", 96, 4, 8, 0.4, False), ("fp16", 24, 3, 8, 0.4, False), ("fp16", 96, 4, 100, 0.1, True)])
+def test_full_sideband_degrades_to_plain_chunks(dn, S, b_r, T, p, single):
+    """A sideband that is too small: the flagged chunks that find no room (the last ones of a (b, h) stream in
+    (row, chunk) order) are stored as plain HQMQ chunks (flag cleared, the quantizer's radius code), so the cache
+    decodes them to the inner quantizer's value, never to zero (the reference never loses an outlier,
+    outlier_aware.py:86).  Planes, counters and the dense decode against the oracle, through every compaction path: the
+    tile-parallel passes (T = 600), the in-order kernel (T = 100), the quantize launch itself (T = 8), and the
+    single-tensor entry points (`single`); then attention over such a cache with both kernels."""
+    import hqmq
+    from hqmq_amd import ops
+    from tests.helpers import assert_attention_close, masked_two_refs
+    dt = DT[dn]
+    B, H, d_h = 2, 2, 128
+    n = d_h // 4
+    inner = hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=S, radius_bits=b_r, device=DEV, seed=5)
+    w = hqmq.with_outlier_extraction(inner)
+    k = kv_input((B, H, T, d_h), dt, seed=S + T, outlier_p=p)
+    v = kv_input((B, H, T, d_h), dt, seed=S + T + 1, outlier_p=p, outlier_gain=(20, 40))
+    cache = w.new_cache(B, T, d_h, dt, 0, sideband_frac=1e-6)
+    cap = cache.K.sb_cap
+    assert cap == 64
+    if single:
+        w.inner._append_one(cache.K, k.to(DEV), 0, 0, None, median_mult=3.0)       # med3x, quantize and compaction as three calls
+        w.inner._append_one(cache.V, v.to(DEV), 0, 1, None, median_mult=3.0)
+    else:
+        w.append(cache, k.to(DEV), v.to(DEV), 0)
+    assert cache.K.overflowed() and cache.V.overflowed()
+    with pytest.raises(Exception):
+        cache.K.check_overflow()
+    for pt, x, kv in ((cache.K, k, 0), (cache.V, v, 1)):
+        Jc = CO.joint_table(TO.secondary_raw(1, H, S, 5)[0, :, kv], dt)
+        want = CO.outlier_quantize(x, Jc, b_r, 3.0)
+        order = want["mask"].reshape(B, H, T * n).long().cumsum(-1).reshape(B, H, T, n)      # 1-based rank in (row, chunk) order
+        kept = want["mask"] & (order <= cap)
+        assert int((want["mask"] & ~kept).sum()) > 0
+        assert torch.equal(pt.flags[:, :, :T].cpu(), CO.pack_flags(kept))
+        rq0 = torch.where(kept, torch.zeros_like(want["rq"]), want["rq"])
+        main, aux = CO.pack_rows(want["idx"], rq0, pt.idx_bits, pt.main_bits, pt.aux_bits)
+        assert torch.equal(pt.main[:, :, :T].cpu(), main)
+        if aux is not None:
+            assert torch.equal(pt.aux[:, :, :T].cpu(), aux)
+        for b in range(B):
+            for h in range(H):
+                sb, _, cnt = CO.pack_sideband(x[b, h], kept[b, h])
+                assert cnt == cap and int(pt.sb_count[b, h]) == int(want["mask"][b, h].sum())       # the counter keeps counting
+                assert bit_equal(pt.sideband[b, h, :cap], sb)
+                assert torch.equal(pt.sb_coord[b, h, :cap].cpu(), CO.pack_coords(kept[b, h]))
+        expect = torch.where(kept.unsqueeze(-1), x.view(B, H, T, n, 4), want["inner_out"].view(B, H, T, n, 4)).reshape(B, H, T, d_h)
+        assert bit_equal(ops.dequant_packed(pt, T, mode=1), expect)
+    Q = torch.randn(B, 4, 1, d_h, generator=torch.Generator().manual_seed(9)).to(dt).to(DEV)
+    refs = masked_two_refs(cache, Q, T)
+    scale = max(1.0, float(refs[0].abs().max()))
+    for generic in (False, True):
+        O = hqmq.fused_attention_packed(Q, cache, force_generic=generic)
+        assert torch.isfinite(O).all()
+        assert_attention_close(O, *refs, base=2e-3 * scale, what=f"generic={generic}")

@@ -185,3 +185,52 @@ def test_range_flag_follows_decode_appends():
     O = hqmq.fused_attention_packed(Q, cache)
     assert torch.isfinite(O.float()).all() and float(O.float().abs().max()) > 10 * float(base.float().abs().max())
     assert torch.equal(O, hqmq.fused_attention_packed(Q, cache, force_generic=True))
+
+
+def test_range_check_after_every_append_leaves_no_window():
+    """RANGE_CHECK_EVERY = 1 (per cache or on the class): the largest scale is read back after every append, so the
+    very first attention call after a token whose scale left [2^-8, 2^15) already takes the guarded kernel; with the
+    default the same call meets the unguarded kernel until the next check (the documented window)."""
+    import hqmq
+    dt = torch.bfloat16
+    q = hqmq.HQMQ(n_layers=1, n_heads=2, secondary_size=96, radius_bits=4, device=DEV)
+    x = kv_input((1, 2, 300, 128), dt, 5).to(DEV)
+    big = (kv_input((1, 2, 1, 128), torch.float32, 7) * 1e7).to(dt).to(DEV)
+    Q = torch.randn(1, 8, 1, 128, generator=torch.Generator().manual_seed(6)).to(dt).to(DEV)
+    outs = {}
+    for every in (1, 256):
+        cache = q.new_cache(1, 512, 128, dt, 0)
+        cache.K.RANGE_CHECK_EVERY = cache.V.RANGE_CHECK_EVERY = every
+        q.append(cache, x, x, 0)
+        q.append(cache, x[:, :, :1], big, 0)
+        assert cache.V.wide_range == (every == 1)
+        outs[every] = hqmq.fused_attention_packed(Q, cache)
+    assert torch.isfinite(outs[1].float()).all()
+    cache.V.refresh_range()                         # the check the default would have run later
+    assert cache.V.wide_range and torch.equal(hqmq.fused_attention_packed(Q, cache), outs[1])
+
+
+def test_outlier_kernels_with_huge_k_and_ordinary_v_stay_on_the_fast_path():
+    """bf16 K of magnitude 1e3 whose outlier chunks (x 50-200) lie beyond the fp16 range, with ordinary V: only V's
+    scales decide the routing (P * V scale is what must stay inside fp16), so the cache stays on the specialised outlier
+    kernels, whose K side keeps the scales in fp32 and feeds the verbatim bf16 chunks to bf16 matrix products (the
+    layout-generic kernel scales them down by the bound of the K scales): finite and within the two-reference bound.
+    (Q is of magnitude 1e-3, so that the scores are of order one: queries are converted to fp16 by both kernels.)"""
+    import hqmq
+    from tests.helpers import masked_two_refs
+    dt = torch.bfloat16
+    B, H, T, d_h = 2, 2, 700, 128
+    w = hqmq.with_outlier_extraction(hqmq.HQMQ(n_layers=1, n_heads=H, secondary_size=24, radius_bits=3, device=DEV), C=3.0)
+    k = (kv_input((B, H, T, d_h), torch.float32, 31, outlier_p=0.02) * 1e3).to(dt).to(DEV)
+    v = kv_input((B, H, T, d_h), dt, 32, outlier_p=0.02, outlier_gain=(5, 10)).to(DEV)
+    cache = w.new_cache(B, T, d_h, dt, 0, sideband_frac=0.25)
+    w.append(cache, k, v, 0)
+    cache.K.check_overflow()
+    assert not cache.V.wide_range
+    assert float(k.float().abs().max()) > 65504.0
+    Q = (torch.randn(B, 8, 1, d_h, generator=torch.Generator().manual_seed(33)) * 1e-3).to(dt).to(DEV)
+    refs = masked_two_refs(cache, Q, T)
+    for generic in (False, True):
+        O = hqmq.fused_attention_packed(Q, cache, force_generic=generic)
+        assert torch.isfinite(O.float()).all()
+        assert_attention_close(O, *refs, base=2e-3 * max(1.0, float(refs[0].abs().max())), what=f"generic={generic}")
