@@ -34,8 +34,8 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the attention kernel as the FETCH_SIZE / WRITE_SIZE counters read them, recorded offline
 # (rocprofv3 --pmc does not run inside this script); known for these contexts only.
-TRAFFIC_FILE = "profiles/attn_fast_kernel_config2_32k_hbm_traffic.txt"
-RECORDED_TRAFFIC_BYTES = {32768: 35.69e6}
+TRAFFIC_FILE = "profiles/attn_lds_kernel_config2_32k_hbm_traffic.txt"
+RECORDED_TRAFFIC_BYTES = {32768: 35.59e6}
 Hq, Hkv, D_H, S, B_R = 32, 8, 128, 96, 4
 
 

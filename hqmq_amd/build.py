@@ -3,6 +3,9 @@ hqmq_amd/libhqmq_bench.so from hqmq_amd/csrc_bench/*.hip: the read-only measurem
 hqmq_amd/bench_ceiling.py time (nothing in the product path loads that one).
 
     python -m hqmq_amd.build            # compile (always) and link
+    python -m hqmq_amd.build --stamps   # also hqmq_amd/libhqmq_amd_stamps.so: the same library with attention_fast.hip compiled
+                                        # with -DHQMQ_STAMPS (time stamps inside the LDS-landing attention kernel, read by
+                                        # hqmq_amd/bench_stamps.py; a measurement build, never loaded by the package itself)
 
 The kernels that decide integers (codeword index, radius code, Med3x mask) are
 compiled with -ffp-contract=off so that every written float operation rounds
@@ -35,7 +38,7 @@ def hipcc() -> str:
     return exe
 
 
-def build(verbose: bool = False) -> Path:
+def build(verbose: bool = False, stamps: bool = False) -> Path:
     cc = hipcc()
     objdir = HERE / "build"
     objdir.mkdir(exist_ok=True)
@@ -72,8 +75,21 @@ def build(verbose: bool = False) -> Path:
         if r.returncode:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("link of the measurement library failed")
+    if stamps:
+        obj = objdir / "attention_fast_stamps.o"
+        cmd = [cc, *COMMON, "-DHQMQ_STAMPS", "-c", str(CSRC / "attention_fast.hip"), "-o", str(obj)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("hipcc failed on attention_fast.hip (stamps)")
+        others = [o for o in objs if o.name != "attention_fast.o"]
+        cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(HERE / "libhqmq_amd_stamps.so"), *map(str, others), str(obj)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("link of the stamps build failed")
     return OUT
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, stamps="--stamps" in sys.argv))

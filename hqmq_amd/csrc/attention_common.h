@@ -218,7 +218,7 @@ __device__ __forceinline__ int v_scale_shift_bits(const PackedDev &v) {
     const uint32_t bits = __builtin_amdgcn_readfirstlane(__builtin_nontemporal_load(v.scale_max));      // wave-uniform
     if (bits == 0u) return 0;                                   // nothing written yet
     const int e = (int)((bits >> 23) & 0xffu) - 127 + 1;        // scale < 2^e
-    return e > 15 ? e - 15 : e < -8 ? e : 0;
+    return e > 15 ? e - 15 : e < -8 ? max(e, -64) : 0;        // at most 2^64 upwards: the fp32 sum of the weights stays finite
 }
 __device__ __forceinline__ float v_scale_shift(const PackedDev &v) { return (float)v_scale_shift_bits(v); }
 

@@ -46,8 +46,11 @@ def _both(L, q, B, Hq, Hkv, T, d_h, dt, seed, n_splits, outliers):
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
     L.check(lib.hqmq_attn_fwd(C.byref(_args(L, Q, O_ref, cache, T, n_splits, ws)), st), "hqmq_attn_fwd")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]          # hipMemGetInfo: sees a hipMalloc inside the library, which torch's counters do not
     L.check(lib.hqmq_attn_fwd_static(C.byref(_args(L, Q, O_new, cache, T, n_splits)), st), "hqmq_attn_fwd_static")
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated during hqmq_attn_fwd_static"
     assert torch.cuda.memory_allocated() == before
     assert ns > 1, "the case must use split partials"
     assert not torch.isnan(O_new.float()).any()
