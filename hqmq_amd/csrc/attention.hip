@@ -396,6 +396,32 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(const flo
     }
 }
 
+// op over all 64 lanes, the result in every lane: quad and row permutations (DPP), then the 16- and 32-lane swaps
+template <class Op>
+__device__ __forceinline__ float wave_reduce(float x, Op op) {
+    auto dpp = [](float v, int ctrl_quad) {
+        const int b = __builtin_bit_cast(int, v);
+        int r;
+        switch (ctrl_quad) {
+            case 0: r = __builtin_amdgcn_update_dpp(0, b, 0xB1, 0xF, 0xF, false); break;     // quad_perm [1,0,3,2]
+            case 1: r = __builtin_amdgcn_update_dpp(0, b, 0x4E, 0xF, 0xF, false); break;     // quad_perm [2,3,0,1]
+            case 2: r = __builtin_amdgcn_update_dpp(0, b, 0x141, 0xF, 0xF, false); break;    // row_half_mirror
+            default: r = __builtin_amdgcn_update_dpp(0, b, 0x140, 0xF, 0xF, false); break;   // row_mirror
+        }
+        return __builtin_bit_cast(float, r);
+    };
+    x = op(x, dpp(x, 0));
+    x = op(x, dpp(x, 1));
+    x = op(x, dpp(x, 2));
+    x = op(x, dpp(x, 3));
+    const uint32_t b = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    x = op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const uint32_t c = __float_as_uint(x);
+    const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return op(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
 // The same merge for the common decode shape (d_h = 128, at most 32 splits, 16-bit output): one wavefront per row and
 // no LDS.  A lane owns two output elements and loads them from all 32 split records at once (8 bytes each, 512 bytes
 // per wavefront and record), together with the (m, l) pair of split (lane & 31): one round trip to memory.  The
@@ -413,13 +439,11 @@ __global__ __launch_bounds__(64) void attn_combine_wave_kernel(const float *__re
 #pragma unroll
     for (int s = 0; s < NS; s++) as[s] = *reinterpret_cast<const float2 *>(base + (size_t)min(s, n_splits - 1) * rec + kPartialHead + 2 * lane);
     if (sl >= n_splits) ml = float2{-INFINITY, 0.f};
-    float M = ml.x;
-#pragma unroll
-    for (int o = 1; o < 32; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
+    // reductions over the wavefront inside the vector unit (lane permutations, no LDS round trips): the upper half
+    // repeats the lower one, so it takes no part in the sum
+    const float M = wave_reduce(ml.x, [](float p, float q) { return fmaxf(p, q); });
     const float w = M > -INFINITY ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;        // -inf - finite = -inf -> 0
-    float L = ml.y * w;
-#pragma unroll
-    for (int o = 1; o < 32; o <<= 1) L += __shfl_xor(L, o);
+    const float L = wave_reduce(lane < 32 ? ml.y * w : 0.f, [](float p, float q) { return p + q; });
     float a0 = 0.f, a1 = 0.f;
 #pragma unroll
     for (int s = 0; s < NS; s++) {
