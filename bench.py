@@ -60,9 +60,11 @@ def build_layers(q, T, dt, dev, n_layers, B=1):
     return caches, queries
 
 
-def graph_us(fn, steps, stream):
+def graph_us(fn, steps, stream, replays=1):
     """Time per step of `steps` calls fn(i) captured in one HIP graph (one untimed replay first); falls back to
-    eager launches when capture is unavailable.  Returns (us per step, used_graph)."""
+    eager launches when capture is unavailable.  replays > 1: the graph is replayed that many times, each replay timed
+    on its own, and the median is returned (the figures beside the headline: the first replays of a workload run
+    before the clocks have settled, by up to 20 % for the long launches).  Returns (us per step, used_graph)."""
     import torch
     graph = None
     try:
@@ -80,15 +82,19 @@ def graph_us(fn, steps, stream):
     except Exception as e:                  # noqa: BLE001
         print(f"graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
         graph = None
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            fn(i)
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps * 1e6, graph is not None
+    times = []
+    for _ in range(max(1, replays)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                fn(i)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) / steps * 1e6)
+    times.sort()
+    return times[len(times) // 2], graph is not None
 
 
 def event_time_us(fn, iters, stream):
@@ -327,6 +333,7 @@ def main():
     us_main_same = kernel_time_us(lambda i, ev: main_kernel(i, ev, False), 192)
     us_launch_interval, _ = graph_us(lambda i: main_kernel(i, None), args.steps, stream)
     us_step_same, _ = graph_us(step_same, args.steps, stream)
+    us_step_settled, _ = graph_us(step, args.steps, stream, replays=9)
     achieved = cache_bytes / (us_main * 1e-6) / 1e9
     # what the memory system allows a launch of this shape: the kernel that only reads the same planes with the same
     # grid, per-wavefront ranges and loads (libhqmq_bench.so: hqmq_bench_read_planes), caches rotating / one cache
@@ -354,6 +361,7 @@ def main():
                    "context": T, "n_splits": n_splits, "hip_graph": used_graph, "layers": NL,
                    "compressed_bytes_per_step": cache_bytes},
         "us_per_step": round(us_step, 2),
+        "us_per_step_median_of_9_replays": round(us_step_settled, 2),
         "pct_of_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
         "max_abs_err_vs_dense_sdpa": max_err,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -408,8 +416,8 @@ def main():
             nl = min(64, max(NL, -(-600_000_000 // (cache_bytes * Tc // T))))
             cs, qs = build_layers(q, Tc, dt, dev, nl)
             ns = ops.pick_splits(1, Hq, Hkv, 1, Tc)
-            us, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[i % nl], cs[i % nl], n_splits=ns, out=outs[0]), args.steps, stream)
-            us1, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[0], cs[0], n_splits=ns, out=outs[0]), args.steps, stream)
+            us, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[i % nl], cs[i % nl], n_splits=ns, out=outs[0]), args.steps, stream, replays=5)
+            us1, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[0], cs[0], n_splits=ns, out=outs[0]), args.steps, stream, replays=5)
             other[str(Tc)] = {"us_per_step": round(us, 2), "GBps": round(cs[0].nbytes(Tc) / us / 1e3, 1), "n_splits": ns,
                               "layers": nl, "same_cache_us_per_step": round(us1, 2)}
             del cs, qs
@@ -418,10 +426,10 @@ def main():
         cs, qs = build_layers(q, T, dt, dev, 2, B=8)
         o8 = torch.empty_like(qs[0])
         ns8 = ops.pick_splits(8, Hq, Hkv, 1, T)
-        us8, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[i % 2], cs[i % 2], n_splits=ns8, out=o8), 48, stream)
+        us8, _ = graph_us(lambda i: hqmq.fused_attention_packed(qs[i % 2], cs[i % 2], n_splits=ns8, out=o8), 48, stream, replays=7)
         result["batch8_steady_state"] = {"us_per_step": round(us8, 2), "GBps": round(cs[0].nbytes(T) / us8 / 1e3, 1),
                                          "pct_of_hbm_roofline": round(100 * cs[0].nbytes(T) / us8 / 1e3 / HBM_PEAK_GBPS, 2),
-                                         "n_splits": ns8, "what": "config 2 shape at batch 8, two caches alternating"}
+                                         "n_splits": ns8, "what": "config 2 shape at batch 8, two caches alternating; median of 7 replays of 48 steps"}
         del cs, qs
         # the one prefill shape the reference publishes (paper App. F: 1.568 ms on an RTX 4090): B = 1, 32 / 8 heads,
         # T = 2048 square causal, d_h 128, s192 with r_qmax = 15, fp16

@@ -475,22 +475,25 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     }
     // Tile offsets of one half-step, in two parts.  The loads (of wave-uniform addresses) are requested two half-steps
-    // ahead; their clamping, which makes the values scalar, happens only when flags_ready has let them through at
-    // the end of a half-step: placed right behind the loads it would wait for them with every later load in flight.
+    // ahead; their clamping happens only when flags_ready has let them through at the end of a half-step: placed right
+    // behind the loads it would wait for them with every later load in flight.
+    // The offsets are read through the constant address space (nothing writes them while this kernel runs), which
+    // makes them scalar loads: as vector loads of one address for all lanes, the six of a half-step took a memory
+    // pipeline slot each and came back through v_readfirstlane (config 4: 10 % of the launch).
+    typedef const int32_t __attribute__((address_space(4))) *const_i32_ptr;
+    const const_i32_ptr k_toff_c = (const_i32_ptr)(uintptr_t)k_toff, v_toff_c = (const_i32_ptr)(uintptr_t)v_toff;
     auto load_flags = [&](int th, FlagTile &f) {
 #pragma unroll
         for (int i = 0; i < 3; i++) {
             const int tc = min((th >> 4) + i, tiles_cap1);
-            f.koff[i] = k_toff[tc];
-            f.voff[i] = v_toff[tc];
+            f.koff[i] = k_toff_c[tc];
+            f.voff[i] = v_toff_c[tc];
         }
     };
     auto flags_ready = [&](int th, FlagTile &f) {
 #pragma unroll
         for (int i = 0; i < 3; i++) {
-            asm volatile("" : "+v"(f.koff[i]), "+v"(f.voff[i]));
-            f.koff[i] = __builtin_amdgcn_readfirstlane(f.koff[i]);       // the same value in every lane: scalar from here on
-            f.voff[i] = __builtin_amdgcn_readfirstlane(f.voff[i]);
+            asm volatile("" : "+s"(f.koff[i]), "+s"(f.voff[i]));        // this is where the scalar loads are waited for
         }
         // tiles not written yet hold INT32_MAX, and so does the slot after the last tile: the count bounds them
 #pragma unroll
