@@ -153,7 +153,9 @@ def run(cfg, steps, emit=True):
     def attend():
         turn[0] += 1
         hqmq.fused_attention_packed(Q, rot[turn[0] % len(rot)], kv_lens=lens_dev, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
-    us = event_us(attend, steps)
+    # the median of three measurements: the first one after the setup above runs before the clocks have settled (config 4:
+    # 288 us against 248 - 265 us for every later one)
+    us = sorted(event_us(attend, steps) for _ in range(3))[1]
     res = {"config": name, "us_per_step": round(us, 2), "compressed_bytes_per_step": step_bytes,
            "GBps": round(step_bytes / us / 1e3, 1), "pct_of_hbm_roofline": round(100 * step_bytes / us / 1e3 / HBM_PEAK_GBPS, 2),
            "n_splits": n_splits, "max_abs_err_vs_dense_fp32": err, "max_abs_ref": ref_max,
@@ -163,7 +165,7 @@ def run(cfg, steps, emit=True):
     if cfg == 4:      # the step of config 4 also quantizes and appends one token per sequence (every context grows by 1)
         pos = lens_dev.clone()
         k1, v1 = k[:, :, :1].contiguous(), v[:, :, :1].contiguous()
-        assert 3 * (steps + 3) + 3 <= T - int(lens.max()), "more timed appends than spare rows"
+        assert 7 * (steps + 3) + 3 <= T - int(lens.max()), "more timed appends than spare rows"
 
         def append():
             w.append(cache, k1, v1, 0, pos=pos)
@@ -172,8 +174,8 @@ def run(cfg, steps, emit=True):
         def step():
             append()
             hqmq.fused_attention_packed(Q, cache, kv_lens=pos, T_kv=T, n_splits=n_splits, out=out, batch_order=order)
-        res["us_per_step_with_append"] = round(event_us(step, steps), 2)
-        res["us_append_only"] = round(event_us(append, steps), 2)
+        res["us_per_step_with_append"] = round(sorted(event_us(step, steps) for _ in range(3))[1], 2)
+        res["us_append_only"] = round(sorted(event_us(append, steps) for _ in range(3))[1], 2)
         # the same step replayed from a HIP graph: what the GPU needs once the ten small launches of an append are
         # not paced by the host (every kernel of the path is capturable: no allocation, no memset, no sync)
         side = torch.cuda.Stream()

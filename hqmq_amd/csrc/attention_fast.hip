@@ -18,6 +18,19 @@
 
 namespace hqmq {
 
+// Time stamps inside the kernels: measurement builds only (-DHQMQ_STAMPS, libhqmq_amd_stamps.so)
+#ifdef HQMQ_STAMPS
+__device__ unsigned long long *g_stamps;
+#define STAMP(i) do { st_[i] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define STAMP(i) do { } while (0)
+#endif
+#ifdef HQMQ_STAMPS
+#define PHASE(i) do { if constexpr (FLAGS) { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); ph_[i] += t_ - tl_; tl_ = t_; } } while (0)
+#else
+#define PHASE(i) do { } while (0)
+#endif
+
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef const uint2 __attribute__((address_space(3))) *lds_u2_ptr;
@@ -335,6 +348,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     constexpr bool kBatchGathers = false;       // see half_step: measured, no gain on any shape (178 against 157 registers)
     constexpr int NH = 1;       // half-steps per prefetched tile: one measures faster than two on every shape
     extern __shared__ uint2 lds_tab[];
+#ifdef HQMQ_STAMPS
+    unsigned long long ph_[8] = {}, tl_ = 0;         // outlier variants: time per phase of the half-steps, summed per wavefront
+    int n_steps_ = 0;
+#endif
     constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
     constexpr int VTAB = vtab_offset(PS), QOFF = q_offset(PS), SELOFF = sel_offset(PS);
     uint2 *ktab = lds_tab, *vtab = lds_tab + VTAB / 8;
@@ -783,6 +800,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 sT[cgi][u] = s;
             }
         }
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(sT[0][0]), "v"(sT[0][1]));
+        PHASE(1);
+#endif
         if constexpr (FLAGS) {
             k_apply(kc, kr, so);
 #pragma unroll
@@ -791,6 +812,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 for (int e = 0; e < 4; e++)
                     sT[0][u][e] = scaled<DT>(sT[0][u][e], e < 2 ? h.ks[u].x : h.ks[u].y, e & 1, so[u][e] * qmaxf);
         }
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(sT[0][0]), "v"(sT[0][1]));
+        PHASE(2);
+#endif
         // the V gathers fly while the softmax below keeps the vector unit busy
         half4 gv[2][CPL];
         half2v rv[2][CPL / 2];
@@ -844,6 +869,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             }
             pp[cgi] = cat8(pT[0], pT[1]);
         }
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(pp[0]));
+        PHASE(3);
+#endif
         // ---- O^T += V^T . P^T, both tiles in one MFMA (the 1/qmax of the radius is applied once, in the epilogue) ----
         if constexpr (kBatchGathers) __builtin_amdgcn_sched_barrier(0);
         half4 av[2][CPL];
@@ -860,7 +889,15 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
             for (int cgi = 0; cgi < NCG; cgi++) acc[cgi][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pp[cgi], acc[cgi][j], 0, 0, 0);
         }
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(acc[0][0]), "v"(acc[0][CPL - 1]));
+        PHASE(4);
+#endif
         if constexpr (FLAGS) v_apply(vc, vr, cat8(pTo[0], pTo[1]));
+#ifdef HQMQ_STAMPS
+        asm volatile("" ::"v"(acc[0][0]), "v"(acc[0][CPL - 1]));
+        PHASE(5);
+#endif
     };
 
     // sideband requests of one half-step
@@ -898,33 +935,53 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             }
         }
     }
-    for (int t0 = t_begin; FLAGS && t0 < t_end; t0 += TS) {
-        FastTile<NW, AB, FLAGS, NH> nxt;
+    if constexpr (FLAGS) {
+        // Outlier variants: one half-step in flight.  Two sets of buffers (tile, sideband entries, tile offsets) take
+        // turns, written out as two half-steps per round of the loop: with one set handed on at the end of every
+        // half-step (cur = nxt) the compiler copied some fifty registers per half-step.
+        // Tile offsets travel two half-steps ahead, sideband entries one (their offsets were requested a step ago); past
+        // the end the current tile is requested again.
+        FastTile<NW, AB, FLAGS, NH> tile_b;
+        KPre<kKPre> k_b = {};
+        VPre<kVPre> v_b = {};
         FlagTile f2 = {};
-        KPre<kKPre> kn = {};
-        VPre<kVPre> vn = {};
-        const bool more = t0 + TS < t_end, more2 = t0 + 2 * TS < t_end;
-        if (FLAGS) {
-            // tile offsets two steps ahead, sideband entries one step ahead (their offsets were requested a step
-            // ago); past the end the current tile is requested again
-            load_super(more ? t0 + TS : t0, nxt);
-            load_flags(more2 ? t0 + 2 * TS : t0, f2);           // made ready at the end of this half-step
-            issue_all(f1, kn, vn);
-        } else if (more) {
-            load_super(t0 + TS, nxt);
-        }
-        half_step(cur.h[0], t0, kc, vc);
-        if (NH == 2 && t0 + 32 < t_end) half_step(cur.h[NH - 1], t0 + 32, kc, vc);
-        if (more) {
-            cur = nxt;
-            if (FLAGS) {
-                kc = kn;
-                vc = vn;
-                flags_ready(more2 ? t0 + 2 * TS : t0, f2);
-                f1 = f2;
+        auto one = [&](int t0, const FastTile<NW, AB, FLAGS, NH> &tile_use, const KPre<kKPre> &k_use, const VPre<kVPre> &v_use,
+                       FastTile<NW, AB, FLAGS, NH> &tile_load, KPre<kKPre> &k_load_to, VPre<kVPre> &v_load_to, const FlagTile &f_use,
+                       FlagTile &f_load) {
+            const bool more = t0 + TS < t_end, more2 = t0 + 2 * TS < t_end;
+#ifdef HQMQ_STAMPS
+            if (tl_ == 0) tl_ = __builtin_amdgcn_s_memrealtime();
+            n_steps_++;
+#endif
+            load_super(more ? t0 + TS : t0, tile_load);
+            load_flags(more2 ? t0 + 2 * TS : t0, f_load);           // made ready at the end of this half-step
+            issue_all(f_use, k_load_to, v_load_to);
+            PHASE(0);
+            half_step(tile_use.h[0], t0, k_use, v_use);
+            if (more) flags_ready(more2 ? t0 + 2 * TS : t0, f_load);
+            PHASE(6);
+            return more;
+        };
+        if (t_begin < t_end) {
+            int t0 = t_begin;
+            while (true) {
+                if (!one(t0, cur, kc, vc, tile_b, k_b, v_b, f1, f2)) break;
+                t0 += TS;
+                if (!one(t0, tile_b, k_b, v_b, cur, kc, vc, f2, f1)) break;
+                t0 += TS;
             }
         }
     }
+#ifdef HQMQ_STAMPS
+    if constexpr (FLAGS) {
+        if (lane == 0 && g_stamps) {
+            unsigned long long *o = g_stamps + ((size_t)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * WV + wave) * 16;
+#pragma unroll
+            for (int i = 0; i < 7; i++) o[i] = ph_[i];
+            o[7] = (unsigned long long)n_steps_;
+        }
+    }
+#endif
 
     // ---- merge the block's waves through LDS: rows of [d_h accumulators, m, l, pad], one column group at a time ----
     constexpr int RS = d_h + 4;
@@ -1016,12 +1073,6 @@ __device__ __forceinline__ void lds_load16_addr(uint32_t lds_base, const uint8_t
 __device__ __forceinline__ uint4v lds_read16(uint32_t a) { return *(lds_u4_ptr)(uintptr_t)a; }
 __device__ __forceinline__ uint2 lds_read8(uint32_t a) { return __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)a); }
 
-#ifdef HQMQ_STAMPS
-__device__ unsigned long long *g_stamps;
-#define STAMP(i) do { st_[i] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define STAMP(i) do { } while (0)
-#endif
 
 constexpr int kLdDepth = 2;
 
