@@ -8,7 +8,11 @@ A step is one fused decode-attention pass of one layer over the compressed cache
 causal=False).  A decode step of a model walks a different layer's cache every time, so the timed steps rotate
 over `--layers` distinct caches (16 x 34.6 MB = 554 MB, more than the 256 MB Infinity Cache and the L2s hold):
 every step reads its cache from HBM.  Inputs (packed caches, queries) are resident in HBM before the timed
-region; the K timed steps are captured in one HIP graph and replayed once between torch.cuda.synchronize().
+region; the K timed steps are captured in one HIP graph and replayed once between two torch.cuda.synchronize()
+(host clock from the replay call to the completion of an event recorded behind the graph, see host_time_s).
+Warm-up: the first 32 of the W warm-up steps are launched one by one, the rest as whole untimed replays of that same
+graph ((W - 32) // K of them, at least one); the default W is 32 + 10 K, about 30 ms of the workload, because the
+first replays after a start run 5 - 10 % slower than every later one (clocks still settling).
 
 One JSON line is printed:
   value        = algorithmic compressed bytes per step / step time (GB/s), whole job on the one GPU, caches
@@ -60,10 +64,10 @@ def build_layers(q, T, dt, dev, n_layers, B=1):
     return caches, queries
 
 
-def graph_us(fn, steps, stream, replays=1):
-    """Time per step of `steps` calls fn(i) captured in one HIP graph (one untimed replay first); falls back to
-    eager launches when capture is unavailable.  replays > 1: the graph is replayed that many times, each replay timed
-    on its own, and the median is returned (the figures beside the headline: the first replays of a workload run
+def graph_us(fn, steps, stream, replays=1, warm_replays=1):
+    """Time per step of `steps` calls fn(i) captured in one HIP graph (`warm_replays` untimed replays first); falls
+    back to eager launches when capture is unavailable.  replays > 1: the graph is replayed that many times, each replay
+    timed on its own, and the median is returned (the figures beside the headline: the first replays of a workload run
     before the clocks have settled, by up to 20 % for the long launches).  Returns (us per step, used_graph)."""
     import torch
     graph = None
@@ -77,24 +81,38 @@ def graph_us(fn, steps, stream, replays=1):
         with torch.cuda.graph(graph):
             for i in range(steps):
                 fn(i)
-        graph.replay()
+        for _ in range(max(1, warm_replays)):
+            graph.replay()
         torch.cuda.synchronize()
     except Exception as e:                  # noqa: BLE001
         print(f"graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
         graph = None
-    times = []
-    for _ in range(max(1, replays)):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
+    def run():
         if graph is not None:
             graph.replay()
         else:
             for i in range(steps):
                 fn(i)
-        torch.cuda.synchronize()
-        times.append((time.perf_counter() - t0) / steps * 1e6)
-    times.sort()
+    times = sorted(host_time_s(run) / steps * 1e6 for _ in range(max(1, replays)))
     return times[len(times) // 2], graph is not None
+
+
+def host_time_s(run):
+    """Host wall time of the GPU work that run() enqueues, between two torch.cuda.synchronize().  The clock stops
+    when an event recorded behind the work reports completion to a polling host: a blocking synchronize returns
+    20 - 40 us after the work has ended (the time the host needs to wake up), which is 1 - 2 us per step when only 20
+    steps are timed."""
+    import torch
+    done = torch.cuda.Event()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run()
+    done.record()
+    while not done.query():
+        pass
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    return t1 - t0
 
 
 def event_time_us(fn, iters, stream):
@@ -244,7 +262,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=192)
-    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=-1, help="untimed warm-up steps (default 32 + 10 x steps)")
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--layers", type=int, default=16, help="distinct caches the timed steps rotate over")
     ap.add_argument("--n-splits", type=int, default=0)
@@ -296,7 +314,11 @@ def main():
         sys.exit(1)
 
     stream = torch.cuda.current_stream()
-    for i in range(args.warmup):
+    if args.warmup < 0:
+        args.warmup = 32 + 10 * args.steps
+    eager_warmup = args.warmup if args.no_graph else min(args.warmup, 32)
+    warm_replays = max(1, (args.warmup - eager_warmup) // max(1, args.steps))
+    for i in range(eager_warmup):
         step(i)
     torch.cuda.synchronize()
     if args.counters:
@@ -311,14 +333,13 @@ def main():
         return
 
     if args.no_graph:
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(i)
-        torch.cuda.synchronize()
-        us_step, used_graph = (time.perf_counter() - t0) / args.steps * 1e6, False
+        def eager():
+            for i in range(args.steps):
+                step(i)
+        us_step, used_graph = host_time_s(eager) / args.steps * 1e6, False
+        warm_replays = 0
     else:
-        us_step, used_graph = graph_us(step, args.steps, stream)
+        us_step, used_graph = graph_us(step, args.steps, stream, warm_replays=warm_replays)
     value = step_bytes / (us_step * 1e-6) / 1e9
 
     # the attention kernel alone (split partials left in the workspace), a pair of HIP events per launch
@@ -349,6 +370,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_steps_run": eager_warmup + warm_replays * args.steps,
         "ms_per_step": round(us_step / 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",

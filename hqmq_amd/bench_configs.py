@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Full-size runs of benchmark configs 3, 4 and 5 on one GPU (config 2 is bench.py's default workload).
 
-    python -m hqmq_amd.bench_configs [--configs 3 4 5] [--steps 50]
+    python -m hqmq_amd.bench_configs [--configs 3 4 5] [--steps 50] [--plain]
+
+--plain builds the same caches without Med3x (no flags, no sideband): what the outlier handling costs on each shape.
 
 For each config: build the packed cache with the HIP quantize path (bulk, Med3x where the config has it), run
 one layer's fused decode-attention step over it, check the output against dense fp32 attention on the
@@ -81,7 +83,7 @@ def dense_check(Q, cache, lens, T):
     return worst, ref_max
 
 
-def run(cfg, steps, emit=True):
+def run(cfg, steps, emit=True, med3x=True):
     if cfg == 3:
         B, Hq, Hkv, d, S, b_r, dt, med = 8, 28, 4, 128, 192, 6, torch.float16, True
         lens, T = None, 32768
@@ -104,6 +106,9 @@ def run(cfg, steps, emit=True):
     else:
         raise SystemExit(f"unknown config {cfg}")
     q = hqmq.HQMQ(n_layers=1, n_heads=Hkv, secondary_size=S, radius_bits=b_r, device=DEV)
+    med = med and med3x
+    if not med:
+        name = name.replace(" + Med3x", " (Med3x off)")
     w = hqmq.with_outlier_extraction(q, C=3.0) if med else q
     cache = w.new_cache(B, T, d, dt, 0, sideband_frac=0.125)
     torch.cuda.synchronize()
@@ -113,8 +118,9 @@ def run(cfg, steps, emit=True):
     e1.record()
     torch.cuda.synchronize()
     quant_ms = e0.elapsed_time(e1)
-    cache.K.check_overflow()
-    cache.V.check_overflow()
+    if med:
+        cache.K.check_overflow()
+        cache.V.check_overflow()
     lens_dev = lens.to(DEV) if lens is not None else None
     if lens is not None:
         cache.crop_(lens_dev)                    # every sequence keeps its own context; the rows behind it are free
@@ -124,7 +130,9 @@ def run(cfg, steps, emit=True):
     # algorithmic bytes of one step: the valid rows of every plane + 8 B per flagged chunk in them
     tokens = int(lens.sum()) if lens is not None else B * T
     row = cache.K.row_bytes()
-    if lens is None:
+    if not med:
+        flagged = 0
+    elif lens is None:
         flagged = int(cache.K.sb_count.sum()) + int(cache.V.sb_count.sum())
     else:
         flagged = 0
@@ -159,7 +167,7 @@ def run(cfg, steps, emit=True):
     res = {"config": name, "us_per_step": round(us, 2), "compressed_bytes_per_step": step_bytes,
            "GBps": round(step_bytes / us / 1e3, 1), "pct_of_hbm_roofline": round(100 * step_bytes / us / 1e3 / HBM_PEAK_GBPS, 2),
            "n_splits": n_splits, "max_abs_err_vs_dense_fp32": err, "max_abs_ref": ref_max,
-           "outlier_rate_K": round(float(cache.K.sb_count.sum()) / (Hkv * tokens * d / 4), 5),      # over the rows kept
+           "outlier_rate_K": round(float(cache.K.sb_count.sum()) / (Hkv * tokens * d / 4), 5) if med else 0.0,      # over the rows kept
            "bulk_quantize_ms_K_and_V": round(quant_ms, 2), "bulk_quantize_GTok_per_s": round(B * T / quant_ms / 1e6, 5),
            "bits_per_value": round(w.bits_per_value(), 3)}
     if cfg == 4:      # the step of config 4 also quantizes and appends one token per sequence (every context grows by 1)
@@ -187,8 +195,9 @@ def run(cfg, steps, emit=True):
         with torch.cuda.graph(graph):
             step()
         res["us_per_step_with_append_graph"] = round(event_us(graph.replay, steps), 2)
-        cache.K.check_overflow()
-        cache.V.check_overflow()
+        if med:
+            cache.K.check_overflow()
+            cache.V.check_overflow()
     res["caches_rotated"] = len(rot)
     if emit:
         print(json.dumps(res), flush=True)
@@ -199,9 +208,10 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--configs", type=int, nargs="+", default=[3, 4, 5])
     ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--plain", action="store_true", help="the same shapes and inputs without Med3x")
     a = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("needs a GPU: the HQMQ kernels have no CPU path")
     for c in a.configs:
-        run(c, a.steps)
+        run(c, a.steps, med3x=not a.plain)
         torch.cuda.empty_cache()
