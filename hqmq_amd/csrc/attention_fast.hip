@@ -25,7 +25,7 @@ __device__ unsigned long long *g_stamps;
 #else
 #define STAMP(i) do { } while (0)
 #endif
-#ifdef HQMQ_STAMPS
+#if defined(HQMQ_STAMPS) && HQMQ_STAMPS + 0 >= 2     // -DHQMQ_STAMPS=2: time per phase of the outlier variants' half-steps (the stamps cost time themselves)
 #define PHASE(i) do { if constexpr (FLAGS) { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); ph_[i] += t_ - tl_; tl_ = t_; } } while (0)
 #else
 #define PHASE(i) do { } while (0)
@@ -351,6 +351,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #ifdef HQMQ_STAMPS
     unsigned long long ph_[8] = {}, tl_ = 0;         // outlier variants: time per phase of the half-steps, summed per wavefront
     int n_steps_ = 0;
+    const unsigned long long t_in_ = __builtin_amdgcn_s_memrealtime();
+    unsigned long long t_loop_ = 0;
 #endif
     constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
     constexpr int VTAB = vtab_offset(PS), QOFF = q_offset(PS), SELOFF = sel_offset(PS);
@@ -369,7 +371,15 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         by = (int)fast_div(r, gridDim.x, p.m_gx);
         bx = (int)(r - (unsigned)by * gridDim.x);
     }
-    const int slot = (int)fast_div((unsigned)bz, (unsigned)p.Hkv, p.m_hkv), hkv = bz - slot * p.Hkv;
+    const int slot = (int)fast_div((unsigned)bz, (unsigned)p.Hkv, p.m_hkv);
+    // Consecutive sequences start with different KV heads: with eight heads (or a multiple) block index modulo 8, and
+    // so the XCD, would otherwise always be the same head, and heads differ in cost (config 4: 20 to 45 sideband
+    // entries per half-step and head, 2.8 to 3.4 us per half-step: the XCD of the densest head finished 20 % after
+    // the others).
+    // (With fewer than eight heads, 8 / Hkv consecutive sequences fill one round of the XCDs and share a rotation.)
+    const int turn = slot >> (p.Hkv == 4 ? 1 : p.Hkv == 2 ? 2 : p.Hkv == 1 ? 3 : 0);
+    int hkv = bz - slot * p.Hkv + (turn - (int)fast_div((unsigned)turn, (unsigned)p.Hkv, p.m_hkv) * p.Hkv);
+    if (hkv >= p.Hkv) hkv -= p.Hkv;
     // The codeword-table loads are the longest dependency chain of the prologue (load, convert, LDS store, barrier)
     // and need nothing but the KV head: they are requested before anything else is worked out.  16-byte loads of two
     // codewords, all unconditional (clamped): straight-line code, exact wait counts.
@@ -600,6 +610,10 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             lds_tab[QOFF / 8 + (c0 + 1) * 16 + col] = uint2{q8[2], q8[3]};
         }
     }
+    // Progress slots of the wavefronts (see `publish` below), behind everything else the loop keeps in LDS
+    const uint32_t prog_base = FLAGS ? (uint32_t)SELOFF + 192u : PS ? 2u * (uint32_t)kPsTabBytes : (uint32_t)kVTabOffset + (uint32_t)p.Vc.K * 8u;
+    typedef int __attribute__((address_space(3))) *lds_i32_ptr;
+    if (threadIdx.x < 16) *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * threadIdx.x) = 0;
     if constexpr (MB == 16 && AB == 3 && IB == 13) {
         if (threadIdx.x < 64) {
             const uint32_t b6 = threadIdx.x;
@@ -900,6 +914,22 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #endif
     };
 
+    // The wavefronts that share a SIMD drift apart: the older one wins every tie for an issue slot, ends up several
+    // half-steps ahead (config 4: 15 us at the end of a block) and leaves the younger to finish alone, with nothing
+    // to overlap its waits.  Every wavefront publishes its position in LDS at the top of a half-step and reads its
+    // SIMD neighbours' (wavefronts w, w + 4, w + 8 share a SIMD); at the end of the half-step it raises its priority
+    // if one of them is ahead and drops it otherwise.
+    int peer_pos = 0;
+    auto publish = [&](int t0) {
+        const int mine = t0 - 32 * wave;        // the same for all wavefronts at the same distance from the block's start
+        *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * (uint32_t)wave) = mine;
+        peer_pos = *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * (uint32_t)((wave + 4) % WV));
+        if constexpr (WV > 8) peer_pos = max(peer_pos, *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * (uint32_t)((wave + 8) % WV)));
+    };
+    auto rebalance = [&](int t0) {
+        if (__builtin_amdgcn_readfirstlane(peer_pos) > t0 - 32 * wave) __builtin_amdgcn_s_setprio(3);
+        else __builtin_amdgcn_s_setprio(0);
+    };
     // sideband requests of one half-step
     auto issue_all = [&](const FlagTile &f, KPre<kKPre> &k, VPre<kVPre> &v) {
         k_issue(f, k);
@@ -921,15 +951,21 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         if (t0 < t_end) {
             while (true) {
                 load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), tc);
+                publish(t0);
                 half_step(cur.h[0], t0, kc, vc);
+                rebalance(t0);
                 t0 += TS;
                 if (t0 >= t_end) break;
                 load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), cur);
+                publish(t0);
                 half_step(tb.h[0], t0, kc, vc);
+                rebalance(t0);
                 t0 += TS;
                 if (t0 >= t_end) break;
                 load_super(readable(t0 + 2 * TS < t_end ? t0 + 2 * TS : t0), tb);
+                publish(t0);
                 half_step(tc.h[0], t0, kc, vc);
+                rebalance(t0);
                 t0 += TS;
                 if (t0 >= t_end) break;
             }
@@ -950,14 +986,16 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                        FlagTile &f_load) {
             const bool more = t0 + TS < t_end, more2 = t0 + 2 * TS < t_end;
 #ifdef HQMQ_STAMPS
-            if (tl_ == 0) tl_ = __builtin_amdgcn_s_memrealtime();
+            if (tl_ == 0) tl_ = t_loop_ = __builtin_amdgcn_s_memrealtime();
             n_steps_++;
 #endif
             load_super(more ? t0 + TS : t0, tile_load);
             load_flags(more2 ? t0 + 2 * TS : t0, f_load);           // made ready at the end of this half-step
             issue_all(f_use, k_load_to, v_load_to);
+            publish(t0);
             PHASE(0);
             half_step(tile_use.h[0], t0, k_use, v_use);
+            rebalance(t0);
             if (more) flags_ready(more2 ? t0 + 2 * TS : t0, f_load);
             PHASE(6);
             return more;
@@ -979,6 +1017,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
 #pragma unroll
             for (int i = 0; i < 7; i++) o[i] = ph_[i];
             o[7] = (unsigned long long)n_steps_;
+            o[8] = t_in_;                   // entry, first half-step, last half-step done (the block's merge follows)
+            o[9] = t_loop_;
+            o[10] = __builtin_amdgcn_s_memrealtime();
+            // where the block ran: HW_ID (bits 8-11 CU, 12 SH, 13-15 SE) and XCC_ID (bits 0-3)
+            o[11] = (unsigned long long)__builtin_amdgcn_s_getreg(((32 - 1) << 11) | 4) |
+                    ((unsigned long long)__builtin_amdgcn_s_getreg(((4 - 1) << 11) | 20) << 32);
+            o[12] = (unsigned long long)b;
         }
     }
 #endif
@@ -1410,7 +1455,8 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st
     if (NCG > 1) grid.y = (grid.y + NCG - 1) / NCG;
     // LDS: K table at 0, V table at kVTabOffset; reused afterwards for the cross-wave merge [wave][16][d_h + 4] floats
     constexpr bool PS = is_prescaled(CPL, MB, AB, IB);
-    size_t shmem = flags ? (size_t)sel_offset(PS) + 9 * 16 : PS ? (size_t)2 * kPsTabBytes : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    size_t shmem = flags ? (size_t)sel_offset(PS) + 192 : PS ? (size_t)2 * kPsTabBytes : (size_t)kVTabOffset + (size_t)p.Vc.K * 8;
+    shmem += 64;        // the wavefronts' progress slots
     const size_t merge = (size_t)WV * 16 * (16 * CPL + 4) * sizeof(float);     // WV >= the wavefronts actually launched
     if (shmem < merge) shmem = merge;
     constexpr int WF = CPL == 4 ? WV : kFastWaves;      // outlier variants fit three wavefronts per SIMD only at d_h 64
