@@ -76,27 +76,6 @@ __device__ __forceinline__ void store_pair(void *tab, int k, uint4v w) {
     else reinterpret_cast<uint4v *>(tab)[k] = pair_to_half<DT>(w);
 }
 
-// The rest of both per-head tables (pairs k0.. of K2 / V2 pairs) -> LDS as fp16, in batches of independent loads.
-template <int DT, int NT, bool F8 = false>
-__device__ __forceinline__ void fill_tables16(void *kdst, const uint4v *ksrc, int Kk2, void *vdst, const uint4v *vsrc, int Kv2, int k_first) {
-    constexpr int U = 3;
-    for (int k0 = k_first + threadIdx.x; k0 < max(Kk2, Kv2); k0 += NT * U) {
-        uint4v tk[U], tv[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int k = k0 + u * NT;
-            tk[u] = ksrc[min(k, Kk2 - 1)];
-            tv[u] = vsrc[min(k, Kv2 - 1)];
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int k = k0 + u * NT;
-            if (k < Kk2) store_pair<DT, F8>(kdst, k, tk[u]);
-            if (k < Kv2) store_pair<DT, F8>(vdst, k, tv[u]);
-        }
-    }
-}
-
 // The parameter block spans several 64-byte lines of the kernel-argument segment, and the prologue reads them one
 // after the other as its address arithmetic proceeds: every first touch of a line is a miss of the scalar cache
 // that the next scalar load waits behind.  One dword of every line, requested together at the very start, turns
@@ -108,6 +87,14 @@ __device__ __forceinline__ void touch_kernargs() {
 #pragma unroll
     for (int i = 0; i < (int)((sizeof(AttnParams) + 63) / 64); i++) t |= ka[16 * i];
     asm volatile("" ::"s"(t));
+}
+
+// One word of a caller's array that no kernel writes while this one runs, at a wave-uniform index: read through the
+// constant address space, i.e. by a scalar load.  (As a vector load it is followed by a wait for every vector load
+// before it: in the prologues below, for the table loads, and once per dependent word.)
+__device__ __forceinline__ int32_t uniform_word(const int32_t *a, int64_t i) {
+    typedef const int32_t __attribute__((address_space(4))) *const_i32_ptr;
+    return ((const_i32_ptr)(uintptr_t)a)[i];
 }
 
 constexpr int kFastWaves = 8;     // wavefronts per block; 12 (three per SIMD) for plain 16+0 caches with long ranges per block
@@ -130,8 +117,8 @@ struct FlagTile {
 template <int NB>
 struct KPre {
     int off[3];
-    uint2 x[NB][2];            // verbatim chunks (raw bits of the cache dtype)
-    uint32_t cc[NB];           // their coordinates: (token & 15) << 8 | chunk, two 16-bit fields
+    uint4v x[NB];              // two verbatim chunks (raw bits of the cache dtype) as loaded, see k_load
+    uint32_t cc[NB];           // their coordinates as loaded: (token & 15) << 8 | chunk, two 16-bit fields
 };
 // V outliers of one half-step: the first NB batches of sixteen entries; lane 16 * grp + col holds entry `col`.
 template <int NB>
@@ -383,7 +370,9 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // The codeword-table loads are the longest dependency chain of the prologue (load, convert, LDS store, barrier)
     // and need nothing but the KV head: they are requested before anything else is worked out.  16-byte loads of two
     // codewords, all unconditional (clamped): straight-line code, exact wait counts.
-    constexpr int FU = 3;
+    // (every pair of the largest table the LDS slots hold, 2560 pairs, in one round of requests: a second round would
+    // be a loop of loads, and the wait at its head covers every request in flight, the first tile's included)
+    constexpr int FU = is_prescaled(CPL, MB, AB, IB) ? (512 + NT - 1) / NT : (kVTabOffset / 16 + NT - 1) / NT;
     const uint4v *ksrc = (const uint4v *)((const uint2 *)p.Kc.joint + hkv * (p.Kc.jsh / 4));
     const uint4v *vsrc = (const uint4v *)((const uint2 *)p.Vc.joint + hkv * (p.Vc.jsh / 4));
     const int Kk2 = p.Kc.K >> 1, Kv2 = p.Vc.K >> 1;        // tables of an even number of codewords (checked at launch)
@@ -394,14 +383,24 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         tk[u] = ksrc[min(k, Kk2 - 1)];
         tv[u] = vsrc[min(k, Kv2 - 1)];
     }
-    const int b = p.batch_order ? min(max(p.batch_order[slot], 0), p.B - 1) : slot;
+#ifdef HQMQ_STAMPS
+    ph_[0] = __builtin_amdgcn_s_memrealtime();      // table loads requested
+#endif
+    const int b = p.batch_order ? min(max(uniform_word(p.batch_order, slot), 0), p.B - 1) : slot;
     const int bh = b * p.Hkv + hkv;
     const int cg0 = by * NCG, sp = bx;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int G = p.G;
     constexpr int n = 4 * CPL, d_h = 16 * CPL;
     const int col = lane & 15, grp = lane >> 4;
-    int kv_end = p.kv_len ? p.kv_len[b] : p.Tkv;
+    // The four per-sequence words go out together, without a branch on the optional pointers (an absent array reads
+    // a word of the kernel arguments instead): one scalar round trip instead of one per word.
+    const int32_t *const spare_word = (const int32_t *)(uintptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+    const int32_t w_len = uniform_word(p.kv_len ? p.kv_len + b : spare_word, 0);
+    const int32_t w_start = uniform_word(p.kv_start ? p.kv_start + b : spare_word, 0);
+    const int32_t w_kcount = uniform_word(FLAGS ? p.Kc.sb_count + bh : spare_word, 0);
+    const int32_t w_vcount = uniform_word(FLAGS ? p.Vc.sb_count + bh : spare_word, 0);
+    int kv_end = p.kv_len ? w_len : p.Tkv;
     kv_end = min(max(kv_end, 0), p.Tkv);
     bool col_ok[NCG];
     int tq[NCG], hq[NCG], col_lim[NCG];
@@ -430,7 +429,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         blk_lim = lim_min = kv_end;         // every column in range sees the whole sequence (a launched block has one)
     }
     // tokens before kv_start[b] are invisible (left padding): the walk starts at the super-tile that holds it
-    const int col_start = p.kv_start ? min(max(p.kv_start[b], 0), blk_lim) : 0;
+    const int col_start = p.kv_start ? min(max(w_start, 0), blk_lim) : 0;
     const int blk_lo = col_start / kSuper * kSuper;
     int per_split = (int)fast_div((unsigned)(blk_lim - blk_lo + p.n_splits - 1), (unsigned)p.n_splits, p.m_splits);
     per_split = (per_split + kSuper - 1) / kSuper * kSuper;
@@ -456,8 +455,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     const int32_t *v_toff = FLAGS ? p.Vc.sb_tile_off + (size_t)bh * tiles_cap : nullptr;
     const uint32_t main_off = (uint32_t)(col * mrb + grp * NB), aux_off = (uint32_t)(col * arb + grp * ABYTES);
     const uint32_t scale_off = (uint32_t)(4 * grp);
-    const int k_count = FLAGS ? (int)min((int64_t)max(p.Kc.sb_count[bh], 0), p.Kc.sb_cap) : 0;
-    const int v_count = FLAGS ? (int)min((int64_t)max(p.Vc.sb_count[bh], 0), p.Vc.sb_cap) : 0;
+    const int k_count = FLAGS ? (int)min((int64_t)max(w_kcount, 0), p.Kc.sb_cap) : 0;
+    const int v_count = FLAGS ? (int)min((int64_t)max(w_vcount, 0), p.Vc.sb_cap) : 0;
     const char *k_side = FLAGS ? (const char *)p.Kc.sideband + (size_t)bh * p.Kc.sb_cap * 8 : nullptr;
     const char *v_side = FLAGS ? (const char *)p.Vc.sideband + (size_t)bh * p.Vc.sb_cap * 8 : nullptr;
     const char *k_coord = FLAGS ? (const char *)p.Kc.sb_coord + (size_t)bh * p.Kc.sb_cap * 2 : nullptr;
@@ -487,20 +486,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     };
 
-    half8 qf[NCG][CPL / 2];
-#pragma unroll
-    for (int cgi = 0; cgi < NCG; cgi++) {
-        const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[cgi] * p.qsh + (int64_t)tq[cgi] * p.qst + grp * CPL * 4;
-#pragma unroll
-        for (int j = 0; j < CPL / 2; j++) {
-            // only the lanes of real columns load (a decode step has G of 16): masked-off lanes cost the memory
-            // pipeline nothing, a clamped load would cost it a full request
-            const half4 z = half4{0, 0, 0, 0};
-            const half4 lo = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j)) : z;
-            const half4 hi = col_ok[cgi] ? chunk_to_half<DT>(*reinterpret_cast<const uint2 *>(qp + 8 * j + 4)) : z;
-            qf[cgi][j] = cat8(lo, hi);
-        }
-    }
     // Tile offsets of one half-step, in two parts.  The loads (of wave-uniform addresses) are requested two half-steps
     // ahead; their clamping happens only when flags_ready has let them through at the end of a half-step: placed right
     // behind the loads it would wait for them with every later load in flight.
@@ -537,22 +522,92 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         }
     };
 
+    // Every load of the loop is issued unconditionally (clamped addresses): a load inside a branch would make the
+    // compiler's wait counts assume it was not issued, and the waits would then cover the next tile's prefetch.
+    // K side.  The sideband entries of a half-step are a contiguous range known from three tile offsets, so no
+    // flag is read: a batch of eight entries is the reduction dimension of one MFMA per tile,
+    //   so[token][column] += sum over entries e of the batch, i < 4:  [token(e) == token] x_e[i] * Q[column][4 chunk(e) + i],
+    // A = the lane's two entries where their token is the lane's row (else zero), B = the Q chunks they meet (LDS).
+    // The lane's two entries are neighbours in the list: one 16-byte load of the chunks (8-byte aligned) and one 4-byte
+    // load of the coordinates (2-byte aligned), at 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked
+    // at launch).  The pair is clamped to the last pair of the list's storage: an entry that is the very last slot of
+    // a full list then arrives in the upper half.  (A wave-uniform branch to an unclamped variant measures slower.)
+    // (The loaded words are kept as they come and put right by k_fix where they are used: touching them here would
+    // make the request wait for its own data, and for every request before it.)
+    auto k_load = [&](int bs, uint4v &x, uint32_t &cc) {
+        const uint32_t ec = min((uint32_t)bs + 2u * (uint32_t)grp, k_cap2);
+        x = *reinterpret_cast<const uint4v_a8 *>(k_side + ec * 8u);
+        cc = *reinterpret_cast<const uint32_a2 *>(k_coord + ec * 2u);
+    };
+    auto k_fix_cc = [&](int bs, uint32_t cc) { return (uint32_t)bs + 2u * (uint32_t)grp > k_cap2 ? cc >> 16 : cc; };
+    auto k_fix_x = [&](int bs, uint4v X, uint2 (&x)[2]) {
+        const bool up = (uint32_t)bs + 2u * (uint32_t)grp > k_cap2;
+        x[0] = uint2{up ? X[2] : X[0], up ? X[3] : X[1]};
+        x[1] = uint2{X[2], X[3]};
+    };
+    auto k_issue = [&](const FlagTile &f, KPre<kKPre> &k) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) k.off[i] = f.koff[i];
+#pragma unroll
+        for (int bq = 0; bq < kKPre; bq++) k_load(k.off[0] + 8 * bq, k.x[bq], k.cc[bq]);
+    };
+    constexpr int kVPre = CPL >= 8 ? 2 : 1;
+    auto v_load = [&](int bs, uint2 &x, uint32_t &cc) {
+        const uint32_t e = min((uint32_t)bs + (uint32_t)col, v_cap1);
+        x = *reinterpret_cast<const uint2 *>(v_side + e * 8u);
+        cc = *reinterpret_cast<const uint16_t *>(v_coord + e * 2u);
+    };
+    auto v_issue = [&](const FlagTile &f, VPre<kVPre> &v) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) v.off[i] = f.voff[i];
+#pragma unroll
+        for (int bq = 0; bq < kVPre; bq++) v_load(v.off[0] + 16 * bq, v.x[bq], v.cc[bq]);
+    };
+    // sideband requests of one half-step
+    auto issue_all = [&](const FlagTile &f, KPre<kKPre> &k, VPre<kVPre> &v) {
+        k_issue(f, k);
+        v_issue(f, v);
+    };
+    KPre<kKPre> kc = {};
+    VPre<kVPre> vc = {};
     FastTile<NW, AB, FLAGS, NH> cur;
     FlagTile f0 = {}, f1 = {};
+    uint2 q_raw[NCG][CPL];      // the query rows as stored
     {
         // unconditional (a wavefront without a range reads a valid tile it never uses): no branch, so the waits for the
         // table loads below count these loads as issued
         const int t_first = min(t_begin, (int)p.t_cap - 32);
         if (FLAGS) load_flags(t_first, f0);
+        // Requests go out in the order their data is used, since they come back in that order and a wait for one is a
+        // wait for all before it: tables (requested at the very start), query rows, first tile, its sideband entries.
+        // All 16 lanes of a row load (columns past the end read column 0 again and are cleared below): unconditional,
+        // so that the waits count them.
+#pragma unroll
+        for (int cgi = 0; cgi < NCG; cgi++) {
+            const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[cgi] * p.qsh + (int64_t)tq[cgi] * p.qst + grp * CPL * 4;
+#pragma unroll
+            for (int j = 0; j < CPL; j++) q_raw[cgi][j] = *reinterpret_cast<const uint2 *>(qp + 4 * j);
+        }
         load_super(t_first, cur);
-        if (FLAGS) load_flags(t_begin + TS < t_end ? t_begin + TS : t_first, f1);        // made ready below
+#ifdef HQMQ_STAMPS
+        ph_[2] = __builtin_amdgcn_s_memrealtime();      // first tile requested
+#endif
+        if constexpr (FLAGS) {
+            // the first half-step's sideband entries are requested here, behind its tile: they travel while the tables
+            // are filled (requested behind the barrier, they were the last thing the first half-step waited for)
+            flags_ready(t_first, f0);
+            issue_all(f0, kc, vc);          // unconditional (clamped addresses): a wavefront without a range reads entries it never uses
+            load_flags(t_begin + TS < t_end ? t_begin + TS : t_first, f1);        // made ready behind the barrier
+        }
     }
+#ifdef HQMQ_STAMPS
+    ph_[1] = __builtin_amdgcn_s_memrealtime();      // the first half-step's entries requested
+#endif
     // Plain variants keep two half-steps in flight; the second is requested right behind the first (both queue
     // behind the table loads, which were requested at the very start).
     auto readable = [&](int t) { return min(t, (int)p.t_cap - 32); };
     FastTile<NW, AB, FLAGS, NH> tb;
     if constexpr (!FLAGS) load_super(readable(t_begin + TS < t_end ? t_begin + TS : t_begin), tb);
-
     half4 ident;                        // B operand of the transposing MFMA: the 16x16 identity
 #pragma unroll
     for (int e = 0; e < 4; e++) ident[e] = (_Float16)((4 * grp + e) == col ? 1.f : 0.f);
@@ -585,7 +640,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                 if (k < Kk2) store_pair<DT, F8>(ktab, k, tk[u]);
                 if (k < Kv2) store_pair<DT, F8>(vtab, k, tv[u]);
             }
-            if (max(Kk2, Kv2) > FU * NT) fill_tables16<DT, NT, F8>(ktab, ksrc, Kk2, vtab, vsrc, Kv2, FU * NT);
         }
     }
     if (FLAGS && threadIdx.x >= 64 && threadIdx.x < 100) {
@@ -595,14 +649,21 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         const uint32_t one = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(float)p.qmax);
         reinterpret_cast<uint32_t *>(lds_tab)[SELOFF / 4 + w] = (row < 8 && (row >> 1) == d) ? one << (16 * (row & 1)) : 0u;
     }
+    half8 qf[NCG][CPL / 2];
+#pragma unroll
+    for (int cgi = 0; cgi < NCG; cgi++) {
+#pragma unroll
+        for (int j = 0; j < CPL / 2; j++) {
+            const half4 z = half4{0, 0, 0, 0};
+            qf[cgi][j] = cat8(col_ok[cgi] ? chunk_to_half<DT>(q_raw[cgi][2 * j]) : z, col_ok[cgi] ? chunk_to_half<DT>(q_raw[cgi][2 * j + 1]) : z);
+        }
+    }
     if (FLAGS && wave == 0) {       // every wavefront of the block has the same 16 columns
 #pragma unroll
         for (int jj = 0; jj < CPL / 2; jj++) {
             uint4v q8 = __builtin_bit_cast(uint4v, qf[0][jj]);
             if constexpr (kBfEntries) {         // the stored bf16 values
-                const uint16_t *qp = (const uint16_t *)p.Q + b * p.qsb + hq[0] * p.qsh + (int64_t)tq[0] * p.qst + grp * CPL * 4;
-                const uint2 lo = col_ok[0] ? *reinterpret_cast<const uint2 *>(qp + 8 * jj) : uint2{0, 0};
-                const uint2 hi = col_ok[0] ? *reinterpret_cast<const uint2 *>(qp + 8 * jj + 4) : uint2{0, 0};
+                const uint2 lo = col_ok[0] ? q_raw[0][2 * jj] : uint2{0, 0}, hi = col_ok[0] ? q_raw[0][2 * jj + 1] : uint2{0, 0};
                 q8 = uint4v{lo.x, lo.y, hi.x, hi.y};
             }
             const int c0 = grp * CPL + 2 * jj;
@@ -620,7 +681,13 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             reinterpret_cast<uint32_t *>(lds_tab)[kAuxTabOffset / 4 + b6] = ((b6 & 7u) << 3) | ((b6 >> 3) << 19) | 0x64006400u;
         }
     }
+#ifdef HQMQ_STAMPS
+    const unsigned long long t_fill_ = __builtin_amdgcn_s_memrealtime();
+#endif
     __syncthreads();
+#ifdef HQMQ_STAMPS
+    const unsigned long long t_bar_ = __builtin_amdgcn_s_memrealtime();
+#endif
 
     // Scores are kept as v = S^T * rs (+ qmax * unscaled outlier part); the softmax argument is c_log2 * v.
     const float c = p.c_log2, qmaxf = (float)p.qmax;
@@ -635,39 +702,17 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     }
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
     const half4 zero_h4 = half4{0, 0, 0, 0};
-    // Every load of the loop is issued unconditionally (clamped addresses): a load inside a branch would make the
-    // compiler's wait counts assume it was not issued, and the waits would then cover the next tile's prefetch.
-    // K side.  The sideband entries of a half-step are a contiguous range known from three tile offsets, so no
-    // flag is read: a batch of eight entries is the reduction dimension of one MFMA per tile,
-    //   so[token][column] += sum over entries e of the batch, i < 4:  [token(e) == token] x_e[i] * Q[column][4 chunk(e) + i],
-    // A = the lane's two entries where their token is the lane's row (else zero), B = the Q chunks they meet (LDS).
-    // The lane's two entries are neighbours in the list: one 16-byte load of the chunks (8-byte aligned) and one 4-byte
-    // load of the coordinates (2-byte aligned), at 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked
-    // at launch).  The pair is clamped to the last pair of the list's storage: an entry that is the very last slot of
-    // a full list then arrives in the upper half.  (A wave-uniform branch to an unclamped variant measures slower.)
-    auto k_load = [&](int bs, uint2 (&x)[2], uint32_t &cc) {
-        const uint32_t e0 = (uint32_t)bs + 2u * (uint32_t)grp, ec = min(e0, k_cap2);
-        const uint4v X = *reinterpret_cast<const uint4v_a8 *>(k_side + ec * 8u);
-        const uint32_t C = *reinterpret_cast<const uint32_a2 *>(k_coord + ec * 2u);
-        const bool up = e0 > k_cap2;
-        x[0] = uint2{up ? X[2] : X[0], up ? X[3] : X[1]};
-        x[1] = uint2{X[2], X[3]};
-        cc = up ? C >> 16 : C;
-    };
-    auto k_issue = [&](const FlagTile &f, KPre<kKPre> &k) {
-#pragma unroll
-        for (int i = 0; i < 3; i++) k.off[i] = f.koff[i];
-#pragma unroll
-        for (int bq = 0; bq < kKPre; bq++) k_load(k.off[0] + 8 * bq, k.x[bq], k.cc[bq]);
-    };
     // the Q chunks the lane's two entries meet (B operand rows), read from LDS well before the batch's MFMAs
     auto k_qrows = [&](uint32_t cc, uint2 (&q)[2]) {
         const uint32_t c0 = cc & (uint32_t)(n - 1), c1 = (cc >> 16) & (uint32_t)(n - 1);
         q[0] = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c0 * 128u + (uint32_t)col * 8u));
         q[1] = __builtin_bit_cast(uint2, *(lds_u2_ptr)(uintptr_t)(QOFF + c1 * 128u + (uint32_t)col * 8u));
     };
-    auto k_batch = [&](const int (&off)[3], int bs, const uint2 (&x)[2], uint32_t cc, const uint2 (&q)[2], float4v (&so)[2]) {
+    auto k_batch = [&](const int (&off)[3], int bs, uint4v x_loaded, uint32_t cc_loaded, const uint2 (&q)[2], float4v (&so)[2]) {
         const int e0 = bs + 2 * grp;
+        uint2 x[2];
+        k_fix_x(bs, x_loaded, x);
+        const uint32_t cc = k_fix_cc(bs, cc_loaded);
         // the row of the half-step (0..31) an entry belongs to; 64 for a slot behind the half-step's entries
         const uint32_t k0 = e0 < off[2] ? ((cc >> 8) & 15u) + (e0 >= off[1] ? 16u : 0u) : 64u;
         const uint32_t k1 = e0 + 1 < off[2] ? ((cc >> 24) & 15u) + (e0 + 1 >= off[1] ? 16u : 0u) : 64u;
@@ -694,17 +739,18 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     };
     auto k_prepare = [&](const KPre<kKPre> &k, KRows &r) {
 #pragma unroll
-        for (int bq = 0; bq < kKPre; bq++) k_qrows(k.cc[bq], r.q[bq]);
+        for (int bq = 0; bq < kKPre; bq++) k_qrows(k_fix_cc(k.off[0] + 8 * bq, k.cc[bq]), r.q[bq]);
     };
     auto k_apply = [&](const KPre<kKPre> &k, const KRows &r, float4v (&so)[2]) {
 #pragma unroll
         for (int bq = 0; bq < kKPre; bq++)
             if (k.off[0] + 8 * bq < k.off[2]) k_batch(k.off, k.off[0] + 8 * bq, k.x[bq], k.cc[bq], r.q[bq], so);
         for (int bs = k.off[0] + 8 * kKPre; bs < k.off[2]; bs += 8) {      // more than the prefetched batches: rare
-            uint2 x[2], q[2];
+            uint4v x;
+            uint2 q[2];
             uint32_t cc;
             k_load(bs, x, cc);
-            k_qrows(cc, q);
+            k_qrows(k_fix_cc(bs, cc), q);
             k_batch(k.off, bs, x, cc, q, so);
         }
     };
@@ -714,18 +760,6 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     //                                            slot (LDS rows), B = the unscaled probabilities of the 32 tokens;
     //   for every chunk position j in use:       X_j^T by the transposing MFMA (A = the entry's chunk in the row
     //   acc[j] += X_j^T . Pg                     group that owns it, else zero), then one 16x16x16 MFMA over entries.
-    constexpr int kVPre = CPL >= 8 ? 2 : 1;
-    auto v_load = [&](int bs, uint2 &x, uint32_t &cc) {
-        const uint32_t e = min((uint32_t)bs + (uint32_t)col, v_cap1);
-        x = *reinterpret_cast<const uint2 *>(v_side + e * 8u);
-        cc = *reinterpret_cast<const uint16_t *>(v_coord + e * 2u);
-    };
-    auto v_issue = [&](const FlagTile &f, VPre<kVPre> &v) {
-#pragma unroll
-        for (int i = 0; i < 3; i++) v.off[i] = f.voff[i];
-#pragma unroll
-        for (int bq = 0; bq < kVPre; bq++) v_load(v.off[0] + 16 * bq, v.x[bq], v.cc[bq]);
-    };
     // the selector row of the lane's entry (A operand of the MFMA that gathers the probabilities), read ahead of use
     auto v_sel = [&](const int (&off)[3], int bs, uint32_t cc) {
         const int e = bs + col;
@@ -930,19 +964,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         if (__builtin_amdgcn_readfirstlane(peer_pos) > t0 - 32 * wave) __builtin_amdgcn_s_setprio(3);
         else __builtin_amdgcn_s_setprio(0);
     };
-    // sideband requests of one half-step
-    auto issue_all = [&](const FlagTile &f, KPre<kKPre> &k, VPre<kVPre> &v) {
-        k_issue(f, k);
-        v_issue(f, v);
-    };
-    KPre<kKPre> kc = {};
-    VPre<kVPre> vc = {};
-    if constexpr (FLAGS) {
-        const int t_first = min(t_begin, (int)p.t_cap - 32);
-        flags_ready(t_first, f0);
-        flags_ready(t_begin + TS < t_end ? t_begin + TS : t_first, f1);
-        if (t_begin < t_end) issue_all(f0, kc, vc);
-    }
+    if constexpr (FLAGS) flags_ready(t_begin + TS < t_end ? t_begin + TS : min(t_begin, (int)p.t_cap - 32), f1);
 
     if constexpr (!FLAGS) {
         // ring of three tile buffers, every load unconditional (past the end the current tile is requested again)
@@ -1024,6 +1046,8 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             o[11] = (unsigned long long)__builtin_amdgcn_s_getreg(((32 - 1) << 11) | 4) |
                     ((unsigned long long)__builtin_amdgcn_s_getreg(((4 - 1) << 11) | 20) << 32);
             o[12] = (unsigned long long)b;
+            o[14] = t_fill_;                // own share of the tables stored, barrier passed
+            o[15] = t_bar_;
         }
     }
 #endif
@@ -1072,6 +1096,12 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
             }
         }
     }
+#ifdef HQMQ_STAMPS
+    if constexpr (FLAGS) {
+        if (lane == 0 && g_stamps)
+            g_stamps[((size_t)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * WV + wave) * 16 + 13] = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1157,10 +1187,10 @@ __global__ __launch_bounds__(WV * 64) void attn_lds_kernel(AttnParams p) {
 #endif
     // the per-sequence words of ragged batches are read before the first request goes out: behind one, the wait for
     // such a word would also wait for every request in flight
-    const int b = order_p ? min(max(order_p[slot], 0), Bn - 1) : slot;
-    int kv_end = len_p ? len_p[b] : Tkv;
+    const int b = order_p ? min(max(uniform_word(order_p, slot), 0), Bn - 1) : slot;
+    int kv_end = len_p ? uniform_word(len_p, b) : Tkv;
     kv_end = min(max(kv_end, 0), Tkv);
-    const int kv_first = start_p ? max(start_p[b], 0) : 0;
+    const int kv_first = start_p ? max(uniform_word(start_p, b), 0) : 0;
     // ---- tables: 1 KB units dealt to the wavefronts round-robin, straight to their place in LDS ----
     {
         const uint32_t kbytes = (uint32_t)KK * 8u, vbytes = (uint32_t)KV * 8u;
