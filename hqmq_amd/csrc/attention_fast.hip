@@ -960,8 +960,9 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
         peer_pos = *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * (uint32_t)((wave + 4) % WV));
         if constexpr (WV > 8) peer_pos = max(peer_pos, *(lds_i32_ptr)(uintptr_t)(prog_base + 4u * (uint32_t)((wave + 8) % WV)));
     };
+    // (A tie goes to the younger wavefront, w >= 4: at equal priority the hardware would give it to the older one.)
     auto rebalance = [&](int t0) {
-        if (__builtin_amdgcn_readfirstlane(peer_pos) > t0 - 32 * wave) __builtin_amdgcn_s_setprio(3);
+        if (__builtin_amdgcn_readfirstlane(peer_pos) + (wave >= 4 ? 1 : 0) > t0 - 32 * wave) __builtin_amdgcn_s_setprio(3);
         else __builtin_amdgcn_s_setprio(0);
     };
     if constexpr (FLAGS) flags_ready(t_begin + TS < t_end ? t_begin + TS : min(t_begin, (int)p.t_cap - 32), f1);
