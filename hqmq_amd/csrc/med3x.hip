@@ -410,10 +410,17 @@ __device__ __forceinline__ void compact_body(const CompactCall &a) {
             if ((row & (kTile - 1)) == 0) sb_tile_off[(size_t)bh * tiles + (row >> 4)] = before;
             int k = before;
             const ST *xr = x + b * xsb + h * xsh + (int64_t)t * xst;
-            uint8_t own[32];                                       // the row's flags as they were (bits may be cleared below)
-            for (int by = 0; by < frb && by < 32; by++) own[by] = fr[by];
-            for (int c = 0; c < n && cnt; c++) {
-                if ((own[c >> 3] >> (c & 7)) & 1) {
+            uint64_t own[4] = {0, 0, 0, 0};                        // the row's flags as they were, in registers (bits may be cleared below)
+            if (cnt) {
+#pragma unroll
+                for (int by = 0; by < 32; by++)
+                    if (by < frb) own[by >> 3] |= (uint64_t)fr[by] << (8 * (by & 7));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                for (uint64_t bits = own[q]; bits; bits &= bits - 1) {
+                    const int c = 64 * q + __builtin_ctzll(bits);
+                    if (c >= n) break;
                     if (k < sb_cap) {
                         ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                         for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
@@ -503,17 +510,23 @@ __global__ void tile_copy_kernel(CompactCall a) {
     const int64_t tiles = (t_cap + kTile - 1) / kTile;
     const int row = row0 + t, tile_row = row & ~(kTile - 1);
     const uint8_t *fr = flag_plane + ((size_t)bh * t_cap + row) * frb;
-    uint8_t mine[32];
-    int own = 0;
-    for (int k = 0; k < frb && k < 32; k++) { mine[k] = fr[k]; own += __popc((uint32_t)mine[k]); }
-    if (!own) return;
+    // the row's flag bits as they are now, in registers (up to 256 chunks): rows whose entries do not fit clear bits
+    // while this one runs
+    uint64_t mine[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int k = 0; k < 32; k++)
+        if (k < frb) mine[k >> 3] |= (uint64_t)fr[k] << (8 * (k & 7));
+    if (!(mine[0] | mine[1] | mine[2] | mine[3])) return;
     int before = a.sb_tile_off[(size_t)bh * tiles + (row >> 4)];
     const uint8_t *f0 = flag_plane + ((size_t)bh * t_cap + tile_row) * frb;
     for (int k = 0; k < (row - tile_row) * frb; k++) before += __popc((uint32_t)f0[k]);
     const ST *xr = x + b * a.xsb + h * a.xsh + (int64_t)t * a.xst;
     int k = before;
-    for (int c = 0; c < n; c++) {
-        if ((mine[c >> 3] >> (c & 7)) & 1) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        for (uint64_t bits = mine[q]; bits; bits &= bits - 1) {
+            const int c = 64 * q + __builtin_ctzll(bits);
+            if (c >= n) break;
             if (k < sb_cap) {
                 ST *dst = sideband + ((size_t)bh * sb_cap + k) * 4;
                 for (int j = 0; j < 4; j++) dst[j] = xr[c * 4 + j];
