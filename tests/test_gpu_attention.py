@@ -98,6 +98,12 @@ CASES = [
     ("s24_r4 + Med3x decode, 12+2 bits", 2, 8, 4, 1, 200, 128, 24, 4, "fp16", True, False, 0, None),
     ("s96_r3 decode, 12+3 bits", 1, 32, 8, 1, 500, 128, 96, 3, "fp16", False, False, 0, None),
     ("s24_r5 square causal prefill, 12+3 bits, two column groups", 1, 32, 8, 160, 160, 128, 24, 5, "fp16", False, True, 0, None),
+    # head counts around the rotation of the KV heads from sequence to sequence (a block's head is not its index
+    # in the grid: (index + sequence slot) mod H_kv, with 8 / H_kv sequences sharing a rotation below eight heads)
+    ("nine sequences, one KV head", 9, 4, 1, 1, 96, 128, 96, 4, "fp16", False, False, 0, None),
+    ("six ragged sequences, two KV heads + Med3x", 6, 4, 2, 1, 150, 128, 24, 3, "bf16", True, False, 0, [150, 7, 64, 33, 150, 99]),
+    ("five sequences, three KV heads", 5, 6, 3, 1, 120, 64, 96, 4, "fp16", False, False, 0, None),
+    ("two sequences, sixteen KV heads", 2, 16, 16, 1, 100, 128, 96, 4, "fp16", False, False, 0, None),
 ]
 
 
