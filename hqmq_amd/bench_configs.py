@@ -83,7 +83,9 @@ def dense_check(Q, cache, lens, T):
     return worst, ref_max
 
 
-def run(cfg, steps, emit=True, med3x=True):
+def setup(cfg, med3x=True):
+    """Inputs, quantizer and filled cache of one config: a dict with B, Hq, Hkv, d, dt, T, lens (CPU int32 or None), lens_dev,
+    k, v, w (the quantizer), cache, name, med (Med3x on), quant_ms (the bulk append)."""
     if cfg == 3:
         B, Hq, Hkv, d, S, b_r, dt, med = 8, 28, 4, 128, 192, 6, torch.float16, True
         lens, T = None, 32768
@@ -124,6 +126,14 @@ def run(cfg, steps, emit=True, med3x=True):
     lens_dev = lens.to(DEV) if lens is not None else None
     if lens is not None:
         cache.crop_(lens_dev)                    # every sequence keeps its own context; the rows behind it are free
+    return dict(B=B, Hq=Hq, Hkv=Hkv, d=d, dt=dt, T=T, lens=lens, lens_dev=lens_dev, k=k, v=v, w=w, cache=cache, name=name, med=med,
+                quant_ms=quant_ms, cfg=cfg)
+
+
+def run(cfg, steps, emit=True, med3x=True):
+    c = setup(cfg, med3x)
+    B, Hq, Hkv, d, dt, T, lens, lens_dev = c["B"], c["Hq"], c["Hkv"], c["d"], c["dt"], c["T"], c["lens"], c["lens_dev"]
+    k, v, w, cache, name, med, quant_ms = c["k"], c["v"], c["w"], c["cache"], c["name"], c["med"], c["quant_ms"]
     Q = torch.randn(B, Hq, 1, d, generator=torch.Generator().manual_seed(7)).to(dt).to(DEV)
     out = torch.empty_like(Q)
     err, ref_max = dense_check(Q, cache, lens, T)

@@ -610,6 +610,7 @@ static int attn_fwd_impl(const hqmq_attn_args *a, void *stream) {
         p.m_hkv = attn_div_magic((uint64_t)a->H_kv, gz);
         p.m_G = attn_div_magic((uint64_t)p.G, gy * 16);
         p.m_splits = attn_div_magic((uint64_t)n_splits, (uint64_t)a->T_kv + (uint64_t)n_splits);
+        if ((gz > 1 && !p.m_gz) || (gx > 1 && !p.m_gx)) p.xcd_remap = 0;      // no multiplier for the renumbering: keep the grid order
     }
     hipStream_t st = (hipStream_t)stream;
     LaunchTiming tm;

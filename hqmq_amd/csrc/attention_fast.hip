@@ -288,9 +288,11 @@ __device__ __forceinline__ void scale_chunks(const half4 (&g)[CPL], const half2v
     for (int j = 0; j < CPL; j++) a[j] = PS ? g[j] : g[j] * r[j >> 1][j & 1];
 }
 
-// x / d through the multiplier the host worked out for d (m = ceil(2^32 / d), exact while x * d < 2^32; 0 where that
-// cannot be promised or d = 1: then the division itself)
-__device__ __forceinline__ unsigned fast_div(unsigned x, unsigned d, unsigned m) { return m ? __umulhi(x, m) : d == 1u ? x : x / d; }
+// x / d through the multiplier the host worked out for d (m = ceil(2^32 / d), exact while x * d < 2^32; m = 0 stands for
+// d = 1: the launcher keeps these kernels for launches where every divisor has its multiplier, see divisors_ready).
+// No division as a fall-back: its expansion, once per use, made the prologue a chain of branches, each with its own
+// re-read of the argument block and a wait for it.
+__device__ __forceinline__ unsigned fast_div(unsigned x, unsigned d, unsigned m) { return m ? __umulhi(x, m) : x; }
 
 __device__ __forceinline__ half8 cat8(half4 x, half4 y) { return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7); }
 
@@ -1086,7 +1088,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
                     a = fmaf(q[e], f, a);
                 }
             }
-            const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
+            const int tq2 = (int)fast_div((unsigned)ci, (unsigned)G, p.m_G), hq2 = hkv * G + (ci - tq2 * G);
             if (p.n_splits == 1) {
                 store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
             } else {
@@ -1444,7 +1446,7 @@ __global__ __launch_bounds__(WV * 64) void attn_lds_kernel(AttnParams p) {
                 a = fmaf(q[e], f, a);
             }
         }
-        const int tq2 = ci / G, hq2 = hkv * G + (ci - tq2 * G);
+        const int tq2 = (int)fast_div((unsigned)ci, (unsigned)G, p.m_G), hq2 = hkv * G + (ci - tq2 * G);
         if (p.n_splits == 1) {
             store_any(p.O, DT, b * p.osb + hq2 * p.osh + (int64_t)tq2 * p.ost + e, l > 0.f ? a * inv_qmax / l : 0.f);
         } else {
@@ -1503,6 +1505,9 @@ static int launch_one(const AttnParams &p, bool flags, dim3 grid, hipStream_t st
 template <int CPL, int DT>
 static int launch_layout(const AttnParams &p, int mb, bool flags, dim3 grid, hipStream_t st, const LaunchTiming &tm, bool *handled) {
     if (p.Kc.K > kVTabOffset / 8 || p.Vc.K > kVTabOffset / 8) return HQMQ_OK;     // tables beyond the fixed LDS slots
+    // the kernels divide by multiplication only (fast_div): sizes for which a multiplier cannot be promised (index times
+    // divisor beyond 2^32: millions of tokens times thousands of splits) stay with the layout-generic kernel
+    if ((p.Hkv > 1 && !p.m_hkv) || (p.G > 1 && !p.m_G) || (p.n_splits > 1 && !p.m_splits)) return HQMQ_OK;
     // the outlier variants keep Q and the selector rows behind a smaller V slot
     if (flags && (p.Kc.K > kFlagsTabMax || p.Vc.K > kFlagsTabMax)) return HQMQ_OK;
     // tables are read two codewords (16 bytes) at a time
