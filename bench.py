@@ -22,8 +22,8 @@ One JSON line is printed:
   cpu_baseline = the CPU restatement of the reference's torch path (decode to dense + SDPA) timed on this host
                  over a token slice of the same cache, and its quantizer on benchmark config 1 in full
 Extra keys: the same step replayed over one cache (resident in the Infinity Cache: an upper bound, labelled),
-the contexts 4k / 8k / 16k, the batch-8 streaming rate, the quantize throughput, configs 3-5 at full size
-(hqmq_amd/bench_configs.py), and the one prefill shape the reference publishes a number for.
+the contexts 4k / 8k / 16k, the batch-8 streaming rate, the quantize throughput, configs 3-5 at full size with and
+without Med3x (hqmq_amd/bench_configs.py), and the one prefill shape the reference publishes a number for.
 """
 import argparse
 import json
@@ -474,7 +474,13 @@ def main():
         result["configs_3_4_5"] = {}
         for cfg in (3, 4, 5):
             r = bench_configs.run(cfg, 30, emit=False)
+            torch.cuda.empty_cache()
+            # the same shape and inputs without Med3x: what the outlier handling costs on this shape
+            plain = bench_configs.run(cfg, 30, emit=False, med3x=False)
+            r["us_per_step_without_med3x"] = plain["us_per_step"]
+            r["med3x_over_plain"] = round(r["us_per_step"] / plain["us_per_step"], 3)
             result["configs_3_4_5"][str(cfg)] = r
+            del plain
             torch.cuda.empty_cache()
     if not args.quick:
         result["config1"] = gpu_config1(dev)
