@@ -289,7 +289,7 @@ __device__ __forceinline__ void scale_chunks(const half4 (&g)[CPL], const half2v
 }
 
 // x / d through the multiplier the host worked out for d (m = ceil(2^32 / d), exact while x * d < 2^32; m = 0 stands for
-// d = 1: the launcher keeps these kernels for launches where every divisor has its multiplier, see divisors_ready).
+// d = 1: the launcher keeps these kernels for launches where every divisor has its multiplier, see launch_layout).
 // No division as a fall-back: its expansion, once per use, made the prologue a chain of branches, each with its own
 // re-read of the argument block and a wait for it.
 __device__ __forceinline__ unsigned fast_div(unsigned x, unsigned d, unsigned m) { return m ? __umulhi(x, m) : x; }
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(WV * 64, WV == 12 ? 3 : 2) void attn_fast_kernel(At
     // load of the coordinates (2-byte aligned), at 32-bit byte offsets from wave-uniform bases (sb_cap < 2^28 is checked
     // at launch).  The pair is clamped to the last pair of the list's storage: an entry that is the very last slot of
     // a full list then arrives in the upper half.  (A wave-uniform branch to an unclamped variant measures slower.)
-    // (The loaded words are kept as they come and put right by k_fix where they are used: touching them here would
+    // (The loaded words are kept as they come and put right by k_fix_x / k_fix_cc where they are used: touching them here would
     // make the request wait for its own data, and for every request before it.)
     auto k_load = [&](int bs, uint4v &x, uint32_t &cc) {
         const uint32_t ec = min((uint32_t)bs + 2u * (uint32_t)grp, k_cap2);
